@@ -172,11 +172,16 @@ class HybridModelConfig:
     streams: int = 1
     conv_taps: int = 0
     embed_scale: float = 1.0
+    # shared-norm arrangement (Legalix): factor on every layer's result
+    # where it joins the residual; layers [start, stop) run `times` times in
+    # a row with the same weights ({"start", "stop", "times"} or None)
+    residual_mult: float = 1.0
+    loop: dict = None
 
     # what the engine asks of any model config
     sliding_window = None
 
-    ARCHITECTURES = ("Gagorax", "Fusolix")
+    ARCHITECTURES = ("Gagorax", "Fusolix", "Legalix")
     MOE_ARCHITECTURES = ("Fusolix",)
 
     @property
@@ -211,7 +216,31 @@ class HybridModelConfig:
             streams=int(cfg.get("streams", 1)),
             conv_taps=int((cfg.get("canon") or {}).get("taps", 0)),
             embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
+            residual_mult=float(cfg.get("residual_mult", 1.0)),
+            loop=cls._read_loop(cfg.get("loop"), len(layers)),
         )
+
+    @staticmethod
+    def _read_loop(loop, n_layers: int):
+        if not loop:
+            return None
+        out = {k: int(loop[k]) for k in ("start", "stop", "times")}
+        if not (0 <= out["start"] < out["stop"] <= n_layers and out["times"] >= 1):
+            raise ValueError(f"loop {loop!r} does not fit {n_layers} layers")
+        return out
+
+    def layer_runs(self) -> tuple:
+        """(layer index of every layer run in execution order, runs that
+        start a pass of the loop)."""
+        n = len(self.layers)
+        if not self.loop:
+            return list(range(n)), []
+        a, b, times = self.loop["start"], self.loop["stop"], self.loop["times"]
+        order, starts = list(range(a)), []
+        for _ in range(times):
+            starts.append(len(order))
+            order += list(range(a, b))
+        return order + list(range(b, n)), starts
 
     def to_dict(self) -> dict:
         out = {"architecture": self.architecture, "vocab": self.vocab_size,
@@ -222,6 +251,12 @@ class HybridModelConfig:
             out.update({"streams": self.streams,
                         "canon": {"taps": self.conv_taps},
                         "embedding": {"scale": self.embed_scale}})
+        if self.architecture == "Legalix":
+            out.pop("logit_scale")
+            out.update({"embedding": {"scale": self.embed_scale},
+                        "residual_mult": self.residual_mult})
+            if self.loop:
+                out["loop"] = dict(self.loop)
         return out
 
     @property
@@ -282,6 +317,38 @@ def _fusolix_preset(width, vocab, pattern, heads, kv_heads, dim, window, pool,
         architecture="Fusolix", vocab_size=vocab, hidden_size=width,
         layers=layers, rms_norm_eps=1e-5, streams=streams, conv_taps=taps,
         embed_scale=1.0)
+
+
+def _legalix_preset(width, vocab, pattern, heads, kv_heads, dim, window,
+                    keep_first, l_heads, l_dim, l_rot, l_vdim, kv_rank, q_rank,
+                    m_heads, m_vdim, m_state, m_groups, ff,
+                    loop=None) -> HybridModelConfig:
+    """pattern: one letter per layer, a (window attention), l (latent
+    attention), m (mamba2); every layer has the dense feed-forward."""
+    layers = []
+    for ch in pattern:
+        if ch == "a":
+            spec = {"type": "attention", "mixer": {
+                "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim,
+                "rot": {"base": 500000.0, "dims": dim}, "scale": dim ** -0.5,
+                "softcap": 50.0,
+                "mask": {"size": window, "keep_first": keep_first}}}
+        elif ch == "l":
+            spec = {"type": "latent_attention", "mixer": {
+                "heads": l_heads, "dim": l_dim, "rot_dim": l_rot,
+                "vdim": l_vdim, "kv_rank": kv_rank, "q_rank": q_rank,
+                "rot": {"base": 10000.0, "dims": l_rot},
+                "scale": (l_dim + l_rot) ** -0.5}}
+        else:
+            spec = {"type": "mamba2", "mixer": {
+                "heads": m_heads, "vdim": m_vdim, "state": m_state,
+                "groups": m_groups, "norm_groups": m_groups, "conv": 4}}
+        spec["mlp"] = {"kind": "dense", "ff": ff}
+        layers.append(spec)
+    return HybridModelConfig(
+        architecture="Legalix", vocab_size=vocab, hidden_size=width,
+        layers=layers, rms_norm_eps=1e-6, embed_scale=1.0,
+        residual_mult=0.5, loop=loop)
 
 
 # Named synthetic configs for benchmarks / tests (random-init weights; no
@@ -568,6 +635,16 @@ PRESET_CONFIGS: dict[str, ModelConfig] = {
         16, 4, 4, 2, 3584),
     "tiny-fusolix": _fusolix_preset(
         128, 512, "dmn", 4, 2, 32, 24, 8, 2, 32, 16, 192, 8, 2, 4, 2, 48),
+    # Legalix at the layer sizes of an ~8B model: 32/8 heads x 128 over a
+    # 1024-token window that keeps the first 4 tokens; 32 latent heads of
+    # 128 plain + 64 rotated dims over a 512-wide cached latent; mamba2 with
+    # 128 heads x 64, state 128 in 8 groups; ff 14336 in every layer
+    "legalix-8b-slice": _legalix_preset(
+        4096, 32000, "malamala", 32, 8, 128, 1024, 4, 32, 128, 64, 128, 512,
+        1536, 128, 64, 128, 8, 14336),
+    "tiny-legalix": _legalix_preset(
+        128, 512, "mal", 4, 2, 32, 24, 3, 4, 16, 8, 24, 32, 40, 4, 16, 8, 2,
+        192, loop={"start": 1, "stop": 3, "times": 2}),
     "tiny-gpu": ModelConfig(  # GPU-test-sized (head_dim 128 kernels)
         architecture="Qwen2ForCausalLM",
         vocab_size=2048,

@@ -25,6 +25,11 @@ _REGISTRY = {
     # input convolution, window/pooled attention beside retention, clamped
     # GLU or group-routed experts (models/hybrid.py StreamBlock)
     "Fusolix": HybridForCausalLM,
+    # layer-list decoder: one tanh norm per layer in front of a mixer and a
+    # GELU GLU side by side; capped window attention that keeps the first
+    # tokens, latent attention, mamba2; a looped run of layers
+    # (models/hybrid.py SharedNormBlock)
+    "Legalix": HybridForCausalLM,
 }
 
 

@@ -1,6 +1,7 @@
 """Feed-forward sublayers of the layer-list decoders, each with its
 constants as constructor parameters:
 
+- GLU: W_down act(W_gate x, W_up x) for the activations of ops.glu_act.
 - ClampedGLU: W_down act(W_gate x, W_up x) with the gate capped from above,
   the up branch clamped on both sides and offset by one:
   g = min(gate, limit), u = clamp(up, -limit, limit),
@@ -30,22 +31,49 @@ from .. import ops
 from .mixers import _param, linear, linear_f32
 
 
-class ClampedGLU(nn.Module):
-    def __init__(self, width: int, ff: int, limit: float, dtype,
-                 alpha: float = 1.702):
+class GLU(nn.Module):
+    """W_down act(W_gate x, W_up x); act is one of ops.glu_act's kinds
+    ("gelu_tanh": gelu_tanh(gate) * up; "swiglu"; "clamped"). Gate and up
+    are one fused GEMM. Without projections of its own it follows the split
+    protocol of models/mixers.py (in_spans, core, out_cols), so that a block
+    can fuse them with its mixer's."""
+
+    def __init__(self, width: int, ff: int, dtype, act: str = "gelu_tanh",
+                 limit: float = 0.0, alpha: float = 1.0,
+                 own_projections: bool = True):
         super().__init__()
-        self.ff, self.limit, self.alpha = ff, float(limit), float(alpha)
-        self.gate_up = _param(2 * ff, width, dtype=dtype)
-        self.down = _param(width, ff, dtype=dtype)
+        self.ff, self.act = ff, act
+        self.limit, self.alpha = float(limit), float(alpha)
+        self.out_cols = ff
+        if own_projections:
+            self.gate_up = _param(2 * ff, width, dtype=dtype)
+            self.down = _param(width, ff, dtype=dtype)
+
+    def in_spans(self) -> list:
+        return [("gate", self.ff, False), ("up", self.ff, False)]
+
+    def extra_weights(self) -> dict:
+        return {}
 
     def weight_map(self) -> dict:
         return {"gate": (self.gate_up, 0), "up": (self.gate_up, self.ff),
                 "down": (self.down, 0)}
 
+    def core(self, p, batch, cache, out, out_scale) -> None:
+        assert out_scale == 1.0
+        ops.glu_act(p, self.act, self.limit, self.alpha, out=out)
+
     def forward(self, h, batch=None, cache=None) -> torch.Tensor:
         gu = linear(h, self.gate_up)
-        return linear(ops.glu_act(gu, "clamped", self.limit, self.alpha),
+        return linear(ops.glu_act(gu, self.act, self.limit, self.alpha),
                       self.down)
+
+
+class ClampedGLU(GLU):
+    def __init__(self, width: int, ff: int, limit: float, dtype,
+                 alpha: float = 1.702):
+        super().__init__(width, ff, dtype, act="clamped", limit=limit,
+                         alpha=alpha)
 
 
 class GroupedMoE(nn.Module):

@@ -32,6 +32,21 @@ GEMM(gate) -> gated_norm_residual [-> GEMM(up|gate) -> gelu_tanh ->
 GEMM(down) -> gated_norm_residual]. The feed-forward's up projection and
 its residual gate read the same row, so they are one fused GEMM.
 
+Legalix's is:
+  - ONE norm per layer, a tanh norm without statistics,
+    h = tanh(alpha x) w + b, read by both sublayers;
+    x += mult * (mixer(h) + ff(h)) (SharedNormBlock)
+  - mixers "attention" (capped scores, window with kept first tokens),
+    "latent_attention", "mamba2"; feed-forward GLU with tanh-GELU
+  - a run of layers may loop: the same weights run `times` passes, each
+    pass with caches and states of its own; every pass starts with
+    x <- W_loop [x | x0], x0 the scaled embedding
+  Kernel plan per layer: residual_tanh_norm (adds the previous layer's
+  result to the fp32 residual and norms, one pass) -> ONE GEMM for every
+  in-projection of the layer [mixer | gate | up] -> mixer kernels and
+  glu_act, each writing its columns of one buffer -> ONE GEMM over
+  [W_o | W_down], whose fp32 accumulation is the sum of both sublayers.
+
 The per-layer cache is a dict of tensors (paged KV for attention, slot
 state for the recurrent mixers and the token shift), allocated by
 allocate_cache() from each mixer's cache_layout(). A sequence that starts at
@@ -51,7 +66,7 @@ from .. import ops
 from ..config import HybridModelConfig
 from ..engine.forward_batch import ForwardBatch
 from ..parallel.comm import get_tp_world_size
-from .feedforward import build_feedforward
+from .feedforward import GLU, build_feedforward
 from .mixers import build_mixer, linear, linear_f32, _param
 
 
@@ -61,7 +76,9 @@ class BlockArrangement:
     gated_residual: bool = True
     # "output": RMS norm on each sublayer's result (HybridBlock);
     # "input": layer norm with bias in front of each sublayer, residual in
-    # weighted copies, short input convolution (StreamBlock)
+    # weighted copies, short input convolution (StreamBlock);
+    # "shared": one tanh norm in front of both sublayers, which run side by
+    # side (SharedNormBlock)
     norm_place: str = "output"
 
 
@@ -69,6 +86,8 @@ ARRANGEMENTS = {
     "Gagorax": BlockArrangement(),
     "Fusolix": BlockArrangement(token_shift=False, gated_residual=False,
                                 norm_place="input"),
+    "Legalix": BlockArrangement(token_shift=False, gated_residual=False,
+                                norm_place="shared"),
 }
 
 
@@ -188,6 +207,67 @@ class StreamBlock(nn.Module):
             yield 2, self.ffn, None
 
 
+class SharedNormBlock(nn.Module):
+    """x += mult * (mixer(h) + ff(h)) with h = tanh(alpha x) w + b: both
+    sublayers are split modules (in_spans / core / out_cols), so the block
+    owns one in-projection [mixer rows | gate | up] and one out-projection
+    [W_o | W_down]; the sum of the two results is the out GEMM's own fp32
+    accumulation."""
+
+    def __init__(self, width: int, spec: dict, eps: float, dtype, arch: str,
+                 ff_act: str = "gelu_tanh"):
+        super().__init__()
+        f32 = torch.float32
+        self.width = width
+        self.mixer = build_mixer(spec["type"], spec["mixer"], width, eps, dtype,
+                                 arch=arch, own_projections=False)
+        mlp = spec.get("mlp")
+        if mlp is not None and mlp.get("kind", "dense") != "dense":
+            raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
+        self.ffn = (GLU(width, mlp["ff"], dtype, act=ff_act,
+                        own_projections=False) if mlp is not None else None)
+        self.parts = [("mix.", self.mixer)] + (
+            [("mlp.", self.ffn)] if self.ffn is not None else [])
+        self.rows = [sum(n for _, n, _ in m.in_spans()) for _, m in self.parts]
+        self.cols = [m.out_cols for _, m in self.parts]
+        self.w_in = _param(sum(self.rows), width, dtype=dtype)
+        self.w_out = _param(width, sum(self.cols), dtype=dtype)
+        self.norm_w = _param(width, dtype=f32)
+        self.norm_b = _param(width, dtype=f32)
+        self.norm_alpha = _param(dtype=f32)
+
+    def weight_map(self) -> dict:
+        m = {"norm1": (self.norm_w, 0), "norm1.b": (self.norm_b, 0),
+             "norm1.alpha": (self.norm_alpha, 0)}
+        row = col = 0
+        for (prefix, part), cols in zip(self.parts, self.cols):
+            for name, n, has_b in part.in_spans():
+                assert not has_b
+                m[prefix + name] = (self.w_in, row)
+                row += n
+            out_name = "o" if prefix == "mix." else "down"
+            m[prefix + out_name] = (self.w_out, 0, col, (self.width, cols))
+            col += cols
+            m.update({prefix + k: v for k, v in part.extra_weights().items()})
+        return m
+
+    def cache_layout(self, block_size: int, dtype) -> dict:
+        return dict(self.mixer.cache_layout(block_size, dtype))
+
+    def forward(self, h, batch: ForwardBatch, cache: dict) -> torch.Tensor:
+        """h: the normed rows; returns mixer(h) + ff(h) in h's dtype."""
+        p = linear(h, self.w_in)
+        buf = torch.empty((h.shape[0], sum(self.cols)), dtype=h.dtype,
+                          device=h.device)
+        row = col = 0
+        for (_, part), rows, cols in zip(self.parts, self.rows, self.cols):
+            part.core(p[:, row:row + rows], batch, cache,
+                      buf[:, col:col + cols], 1.0)
+            row += rows
+            col += cols
+        return linear(buf, self.w_out)
+
+
 class HybridForCausalLM(nn.Module):
     supports_float32 = True
     has_sequence_state = True  # engine: state slots, no prefix reuse
@@ -207,10 +287,22 @@ class HybridForCausalLM(nn.Module):
                 StreamBlock(W, spec, cfg.streams, cfg.conv_taps,
                             cfg.rms_norm_eps, dtype)
                 for spec in cfg.layers)
+        elif arr.norm_place == "shared":
+            self.layers = nn.ModuleList(
+                SharedNormBlock(W, spec, cfg.rms_norm_eps, dtype,
+                                cfg.architecture)
+                for spec in cfg.layers)
         else:
             self.layers = nn.ModuleList(
                 HybridBlock(W, spec, cfg.rms_norm_eps, dtype, arr)
                 for spec in cfg.layers)
+        # layer runs in execution order (a looped layer once per pass, each
+        # run with a cache of its own) and the runs that open a pass
+        if hasattr(cfg, "layer_runs"):
+            self.run_order, loop_starts = cfg.layer_runs()
+        else:
+            self.run_order, loop_starts = list(range(len(self.layers))), []
+        self.loop_starts = frozenset(loop_starts)
         self.final_norm = _param(W, dtype=torch.float32)
         self.head = _param(cfg.vocab_size, W, dtype=dtype)
         self._wmap = {"embed": (self.embed, 0), "head": (self.head, 0),
@@ -220,6 +312,14 @@ class HybridForCausalLM(nn.Module):
             self._wmap["final.norm.b"] = (self.final_norm_b, 0)
             self.register_buffer("sum_w", torch.ones(cfg.streams),
                                  persistent=False)
+        if arr.norm_place == "shared":
+            self.final_norm_b = _param(W, dtype=torch.float32)
+            self.final_norm_alpha = _param(dtype=torch.float32)
+            self._wmap["final.norm.b"] = (self.final_norm_b, 0)
+            self._wmap["final.norm.alpha"] = (self.final_norm_alpha, 0)
+            if self.loop_starts:
+                self.loop_in = _param(W, 2 * W, dtype=dtype)
+                self._wmap["loop.in"] = (self.loop_in, 0)
         for i, layer in enumerate(self.layers):
             for k, v in layer.weight_map().items():
                 self._wmap[f"l{i}.{k}"] = v
@@ -228,7 +328,10 @@ class HybridForCausalLM(nn.Module):
 
     # ------------------------------------------------------------ cache
     def cache_layout(self, block_size: int) -> list:
-        return [layer.cache_layout(block_size, self.dtype) for layer in self.layers]
+        """One dict per layer RUN: every pass of a looped layer has pages
+        and state of its own."""
+        return [self.layers[i].cache_layout(block_size, self.dtype)
+                for i in self.run_order]
 
     def kv_block_bytes(self, block_size: int) -> int:
         total = 0
@@ -262,6 +365,8 @@ class HybridForCausalLM(nn.Module):
         """fp32 logits for batch.logits_indices rows (all rows if None)."""
         if self.arr.norm_place == "input":
             return self._forward_streams(batch, caches)
+        if self.arr.norm_place == "shared":
+            return self._forward_shared(batch, caches)
         x = self.embed[batch.input_ids].float()
         for i, layer in enumerate(self.layers):
             layer(x, batch, caches[i], self.dtype)
@@ -309,6 +414,44 @@ class HybridForCausalLM(nn.Module):
         if batch.logits_indices is not None:
             n = n[batch.logits_indices]
         return linear_f32(n.to(dtype), self.head) * cfg.logit_scale
+
+    def _forward_shared(self, batch: ForwardBatch, caches: list) -> torch.Tensor:
+        """Shared-norm arrangement: a layer's result waits until the kernel
+        that norms the next layer's input adds it to the residual, so each
+        layer costs one pass over the fp32 rows."""
+        cfg, dtype = self.cfg, self.dtype
+        mult = cfg.residual_mult
+        x = self.embed[batch.input_ids].float()
+        if cfg.embed_scale != 1.0:
+            x *= cfg.embed_scale
+        cat = None
+        if self.loop_starts:
+            # [x | x0] rows of the loop's input projection; the right half
+            # is written once
+            W = cfg.hidden_size
+            cat = torch.empty((x.shape[0], 2 * W), dtype=dtype, device=x.device)
+            cat[:, W:] = x
+        y = None
+        for run, i in enumerate(self.run_order):
+            layer = self.layers[i]
+            if run in self.loop_starts:
+                ops.residual_tanh_norm(x, y, mult, None, None, None, dtype,
+                                       xa=cat[:, :cfg.hidden_size])
+                x = linear_f32(cat, self.loop_in)
+                y = None
+            h = ops.residual_tanh_norm(x, y, mult, layer.norm_alpha,
+                                       layer.norm_w, layer.norm_b, dtype)
+            y = layer(h, batch, caches[run])
+            if self.residual_tap is not None:
+                ops.residual_tanh_norm(x, y, mult, None, None, None, dtype)
+                y = None
+                self.residual_tap(run, x)
+        if batch.logits_indices is not None:
+            x = x[batch.logits_indices]
+            y = y[batch.logits_indices] if y is not None else None
+        n = ops.residual_tanh_norm(x, y, mult, self.final_norm_alpha,
+                                   self.final_norm, self.final_norm_b, dtype)
+        return linear_f32(n, self.head) * cfg.logit_scale
 
     # ------------------------------------------------------------ weights
     @staticmethod
@@ -378,8 +521,14 @@ class HybridForCausalLM(nn.Module):
                 return torch.randn(shape, generator=g, device=dev,
                                    dtype=torch.float32) * std
 
-            if leaf.endswith("norm") or leaf in ("norm1", "norm2"):
+            if leaf.endswith(".alpha"):
+                w = 0.5 + 0.5 * torch.rand(shape, generator=g, device=dev)
+            elif leaf.endswith("norm") or leaf in ("norm1", "norm2"):
                 w = 1.0 + rn(0.1)
+            elif leaf == "mix.dt_bias":
+                w = rn(0.5) - 1.0
+            elif leaf == "mix.sink":
+                w = rn(1.0)
             elif leaf.startswith("canon"):
                 w = rn(0.3)
             elif leaf.startswith("hc") and leaf.endswith(".in"):

@@ -19,8 +19,20 @@ constructor parameters so that more than one design can use it:
 - ParallelMixer: two of the above fed the same input, as ONE
   in-projection GEMM and ONE out-projection GEMM over the concatenated
   (pre-scaled) head outputs.
+- SinkRotaryAttention also takes tanh-capped scores (softcap) and a sliding
+  window that keeps the first keys of the sequence visible (window,
+  keep_first); without own projections it is a split mixer too.
+- LatentAttention: queries and keys/values through low-rank latents; the
+  cache holds one normed latent and one rotated key part per token, shared
+  by all heads, and the per-head up-projections are applied to the query
+  and to the attention result instead of to every cached token; a learned
+  per-head sink in the softmax.
+- Mamba2Mixer: short causal convolution over [x | B | C], one scalar decay
+  per head and token, an [state x vdim] fp32 state per head and sequence,
+  silu gate, RMS norm in equal groups of channels.
 
-The last three are "split" mixers: they name the rows of their
+WindowPoolAttention, RetentionMixer, LatentAttention and Mamba2Mixer are
+"split" mixers: they name the rows of their
 in-projection (in_spans) and the columns of their out-projection
 (out_cols) and do everything between in core(), so that a parent can fuse
 the projections of several of them; alone, SplitMixer.forward runs the
@@ -87,7 +99,7 @@ def step_chunks(batch: ForwardBatch, device):
 
 
 def _param(*shape, dtype):
-    return nn.Parameter(torch.zeros(*shape, dtype=dtype), requires_grad=False)
+    return nn.Parameter(torch.zeros(shape, dtype=dtype), requires_grad=False)
 
 
 def rotary_inv_freq(base: float, ndims: int) -> torch.Tensor:
@@ -104,15 +116,26 @@ class SinkRotaryAttention(nn.Module):
     def __init__(self, width: int, heads: int, kv_heads: int, dim: int,
                  vdim: int, scale: float, rot_base: float, rot_dims: int,
                  eps: float, dtype, qk_norm: bool = True, sink: bool = True,
-                 rotate_values: bool = True, interleaved: bool = True):
+                 rotate_values: bool = True, interleaved: bool = True,
+                 softcap: float = 0.0, window: int = 0, keep_first: int = 0,
+                 own_projections: bool = True):
         super().__init__()
         assert heads % kv_heads == 0 and rot_dims % 2 == 0 and rot_dims <= dim
         assert not rotate_values or vdim % 2 == 0
         self.H, self.G, self.D, self.V = heads, kv_heads, dim, vdim
         self.scale, self.eps = float(scale), eps
         self.sink, self.interleaved = sink, interleaved
-        self.qkv = _param(heads * dim + kv_heads * (dim + vdim), width, dtype=dtype)
-        self.o = _param(width, heads * vdim, dtype=dtype)
+        # scores c tanh(s / c); row i sees key j <= i iff i - j < window or
+        # j < keep_first (0: plain causal)
+        self.softcap, self.window = float(softcap), int(window)
+        self.keep_first = int(keep_first)
+        self.masked = self.softcap > 0 or self.window > 0
+        assert not (self.masked and rotate_values)
+        self.out_cols = heads * vdim
+        if own_projections:
+            self.qkv = _param(heads * dim + kv_heads * (dim + vdim), width,
+                              dtype=dtype)
+            self.o = _param(width, heads * vdim, dtype=dtype)
         self.q_norm = _param(dim, dtype=torch.float32) if qk_norm else None
         self.k_norm = _param(dim, dtype=torch.float32) if qk_norm else None
         self.register_buffer("inv_freq_qk", rotary_inv_freq(rot_base, rot_dims),
@@ -122,13 +145,20 @@ class SinkRotaryAttention(nn.Module):
             rotary_inv_freq(rot_base, vdim) if rotate_values else None,
             persistent=False)
 
+    def in_spans(self) -> list:
+        return [("q", self.H * self.D, False), ("k", self.G * self.D, False),
+                ("v", self.G * self.V, False)]
+
+    def extra_weights(self) -> dict:
+        if self.q_norm is None:
+            return {}
+        return {"q.norm": (self.q_norm, 0), "k.norm": (self.k_norm, 0)}
+
     def weight_map(self) -> dict:
         H, G, D, V = self.H, self.G, self.D, self.V
         m = {"q": (self.qkv, 0), "k": (self.qkv, H * D),
              "v": (self.qkv, H * D + G * D), "o": (self.o, 0)}
-        if self.q_norm is not None:
-            m["q.norm"] = (self.q_norm, 0)
-            m["k.norm"] = (self.k_norm, 0)
+        m.update(self.extra_weights())
         return m
 
     def cache_layout(self, block_size: int, dtype) -> dict:
@@ -160,10 +190,43 @@ class SinkRotaryAttention(nn.Module):
                 self.D, q.device)
         return batch.tile_cache[key]
 
+    def core(self, p, batch: ForwardBatch, cache: dict, out, out_scale) -> None:
+        """p: rows of the in-projection [q | k | v]; writes the head outputs,
+        times out_scale, into out [T, H * V] (rows may be strided)."""
+        H, G, D, V = self.H, self.G, self.D, self.V
+        q = p[:, :H * D].unflatten(-1, (H, D))
+        k = p[:, H * D:(H + G) * D].unflatten(-1, (G, D))
+        v = p[:, (H + G) * D:(H + G) * D + G * V].unflatten(-1, (G, V))
+        q = ops.qk_norm_rope_cache(
+            q, k, v, self.q_norm, self.k_norm, self.eps, batch.positions,
+            self.inv_freq_qk, self.inv_freq_v, cache["k"], cache["v"],
+            batch.slot_mapping, self.interleaved)
+        if self.masked:
+            ops.attention_sink_paged(
+                q, cache["k"], cache["v"], batch.block_tables, batch.seq_lens,
+                batch.cu_seqlens, batch.token_seq, self.scale, self.sink,
+                None, self.interleaved, batch.max_q_len, batch.positions,
+                softcap=self.softcap, window=self.window,
+                keep_first=self.keep_first, out=out.unflatten(-1, (H, V)),
+                out_scale=out_scale)
+            return
+        res = ops.attention_sink_paged(
+            q, cache["k"], cache["v"], batch.block_tables, batch.seq_lens,
+            batch.cu_seqlens, batch.token_seq, self.scale, self.sink,
+            self.inv_freq_v, self.interleaved, batch.max_q_len,
+            batch.positions, self._tiles(batch, q))
+        if out_scale != 1.0:
+            res = res * out_scale
+        out.copy_(res.view(p.shape[0], H * V))
+
     def forward(self, xs, batch: ForwardBatch, cache: dict) -> torch.Tensor:
         T = xs.shape[0]
         H, G, D, V = self.H, self.G, self.D, self.V
         qkv = linear(xs, self.qkv)
+        if self.masked:
+            out = torch.empty((T, H * V), dtype=xs.dtype, device=xs.device)
+            self.core(qkv, batch, cache, out, 1.0)
+            return linear(out, self.o)
         q = qkv[:, :H * D].unflatten(-1, (H, D))
         k = qkv[:, H * D:(H + G) * D].unflatten(-1, (G, D))
         v = qkv[:, (H + G) * D:].unflatten(-1, (G, V))
@@ -307,7 +370,12 @@ class SplitMixer(nn.Module):
         m["o"] = (self.w_out, 0)
         if self.b_out is not None:
             m["o.b"] = (self.b_out, 0)
+        m.update(self.extra_weights())
         return m
+
+    def extra_weights(self) -> dict:
+        """Tensors besides the projections the parent may fuse."""
+        return {}
 
     def forward(self, xs, batch: ForwardBatch, cache: dict) -> torch.Tensor:
         p = linear(xs, self.w_in, self.b_in)
@@ -413,6 +481,149 @@ class RetentionMixer(SplitMixer):
         ops.head_norm_gate(o.view(T, H * V), g, self.eps, H, out, out_scale)
 
 
+class LatentAttention(SplitMixer):
+    """Attention through low-rank latents. Per row: c_q = rmsnorm(W_dq h),
+    q = W_uq c_q, laid out per head as [dim plain | rot_dim rotated];
+    W_dkv h = [kv_rank | rot_dim]: the first part RMS-normed is the latent c,
+    the second, rotated (interleaved pairs), is one key part shared by all
+    heads. Keys are [W_uk c | shared part], values W_uv c, causal softmax
+    with a learned per-head sink in the denominator.
+
+    Only [c | rotated part] is cached, one row per token ("ckv", one
+    key/value head). The up-projections move to the other side of the
+    products: q_h' = W_uk,h^T q_h,plain (length kv_rank), so the score is
+    q_h' . c + q_h,rot . k_rot and the softmax-weighted sum of latents is
+    multiplied by W_uv,h afterwards. The attention kernels therefore see H
+    query heads of size kv_rank + rot_dim on ONE key/value head whose value
+    is the first kv_rank columns of its key row."""
+
+    def __init__(self, width: int, heads: int, dim: int, rot_dim: int,
+                 vdim: int, kv_rank: int, q_rank: int, scale: float,
+                 rot_base: float, eps: float, dtype,
+                 own_projections: bool = True):
+        super().__init__()
+        assert rot_dim % 2 == 0
+        self.H, self.D, self.R, self.V = heads, dim, rot_dim, vdim
+        self.rank, self.q_rank = kv_rank, q_rank
+        self.scale, self.eps = float(scale), eps
+        self.out_cols = heads * vdim
+        f32 = torch.float32
+        self.dq_norm = _param(q_rank, dtype=f32)
+        self.dkv_norm = _param(kv_rank, dtype=f32)
+        self.uq = _param(heads * (dim + rot_dim), q_rank, dtype=dtype)
+        # per head [dim, kv_rank] and [vdim, kv_rank], heads stacked by rows
+        self.uk = _param(heads * dim, kv_rank, dtype=dtype)
+        self.uv = _param(heads * vdim, kv_rank, dtype=dtype)
+        self.sink = _param(heads, dtype=f32)
+        self.register_buffer("inv_freq", rotary_inv_freq(rot_base, rot_dim),
+                             persistent=False)
+        if own_projections:
+            self._make_projections(width, dtype)
+
+    def in_spans(self) -> list:
+        return [("dq", self.q_rank, False), ("dkv", self.rank + self.R, False)]
+
+    def extra_weights(self) -> dict:
+        return {"dq.norm": (self.dq_norm, 0), "dkv.norm": (self.dkv_norm, 0),
+                "uq": (self.uq, 0), "sink": (self.sink, 0),
+                "uk": (self.uk, 0), "uv": (self.uv, 0)}
+
+    def cache_layout(self, block_size: int, dtype) -> dict:
+        return {"ckv": ("paged", (1, block_size, self.rank + self.R), dtype)}
+
+    def core(self, p, batch: ForwardBatch, cache: dict, out, out_scale) -> None:
+        T = p.shape[0]
+        H, D, R, V, rank = self.H, self.D, self.R, self.V, self.rank
+        ckv = cache["ckv"]
+        cq = ops.latent_prepare(
+            p[:, :self.q_rank], p[:, self.q_rank:self.q_rank + rank + R],
+            self.dq_norm, self.dkv_norm, self.eps, batch.positions,
+            self.inv_freq, ckv, batch.slot_mapping)
+        q = linear(cq, self.uq).view(T, H, D + R)
+        # [H, T, D] x [H, D, rank]: the key up-projection applied to q
+        q_abs = torch.bmm(q[..., :D].transpose(0, 1),
+                          self.uk.view(H, D, rank))
+        qf = torch.empty((T, H, rank + R), dtype=p.dtype, device=p.device)
+        ops.latent_query(q, q_abs, batch.positions, self.inv_freq, qf)
+        o_lat = ops.attention_sink_paged(
+            qf, ckv, ckv[..., :rank], batch.block_tables, batch.seq_lens,
+            batch.cu_seqlens, batch.token_seq, self.scale, False, None, True,
+            batch.max_q_len, batch.positions, sink_w=self.sink)
+        # [H, T, rank] x [H, rank, V]: the value up-projection
+        o = torch.bmm(o_lat.transpose(0, 1),
+                      self.uv.view(H, V, rank).transpose(1, 2))
+        if out_scale != 1.0:
+            o = o * out_scale
+        out.unflatten(-1, (H, V)).copy_(o.transpose(0, 1))
+
+
+class Mamba2Mixer(SplitMixer):
+    """In-projection rows [z: inner | x: inner | B: G*N | C: G*N | dt: P]
+    with inner = P * vdim. [x | B | C] pass a causal depthwise convolution
+    (taps per channel, bias) and silu; dt = softplus(dt + dt_bias); head h
+    (group h // (P / G)) keeps S_h (N x vdim, fp32):
+    S_h <- exp(-exp(A_log_h) dt_h) S_h + dt_h B x_h^T,
+    y_h = S_h^T C + D_h x_h. Then y * silu(z), unit RMS in norm_groups equal
+    parts of the channels, times the norm weight."""
+
+    def __init__(self, width: int, heads: int, vdim: int, state: int,
+                 groups: int, norm_groups: int, conv: int, eps: float, dtype,
+                 own_projections: bool = True):
+        super().__init__()
+        inner = heads * vdim
+        assert heads % groups == 0 and inner % norm_groups == 0
+        self.P, self.V, self.N, self.G = heads, vdim, state, groups
+        self.inner, self.norm_groups = inner, norm_groups
+        self.taps, self.eps = conv, eps
+        self.ch = inner + 2 * groups * state  # convolved channels
+        self.out_cols = inner
+        f32 = torch.float32
+        self.conv_w = _param(self.ch, conv, dtype=f32)
+        self.conv_b = _param(self.ch, dtype=f32)
+        self.dt_bias = _param(heads, dtype=f32)
+        self.A_log = _param(heads, dtype=f32)
+        self.D = _param(heads, dtype=f32)
+        self.norm = _param(inner, dtype=f32)
+        self.register_buffer("rate", torch.zeros(heads, dtype=f32),
+                             persistent=False)
+        self.register_buffer("conv_w_t", torch.zeros(conv, self.ch, dtype=f32),
+                             persistent=False)
+        if own_projections:
+            self._make_projections(width, dtype)
+
+    def in_spans(self) -> list:
+        return [("in", 2 * self.inner + 2 * self.G * self.N + self.P, False)]
+
+    def extra_weights(self) -> dict:
+        return {"conv": (self.conv_w, 0), "conv.b": (self.conv_b, 0),
+                "dt_bias": (self.dt_bias, 0), "A_log": (self.A_log, 0),
+                "D": (self.D, 0), "norm": (self.norm, 0)}
+
+    def finish_loading(self) -> None:
+        self.rate.copy_(torch.exp(self.A_log.data.float()))
+        self.conv_w_t.copy_(self.conv_w.data.t())
+
+    def cache_layout(self, block_size: int, dtype) -> dict:
+        out = {"ssm": ("slot", (self.P, self.N, self.V), torch.float32)}
+        if self.taps > 1:
+            out["conv"] = ("slot", (self.taps - 1, self.ch), torch.float32)
+        return out
+
+    def core(self, p, batch: ForwardBatch, cache: dict, out, out_scale) -> None:
+        inner, ch = self.inner, self.ch
+        xbc = ops.causal_conv_silu(
+            p[:, inner:inner + ch], self.conv_w, self.conv_b, cache.get("conv"),
+            batch.cu_seqlens, batch.seq_lens, batch.state_slots,
+            batch.token_seq, self.conv_w_t)
+        y = ops.mamba2_scan(
+            xbc, p[:, inner + ch:inner + ch + self.P], self.dt_bias, self.rate,
+            self.D, cache["ssm"], batch.cu_seqlens, batch.seq_lens,
+            batch.state_slots, self.P, self.V, self.N, self.G,
+            batch.max_q_len, step_chunks(batch, p.device))
+        ops.gate_group_norm(y, p[:, :inner], self.norm, self.norm_groups,
+                            self.eps, out, out_scale)
+
+
 class ParallelMixer(nn.Module):
     """left_scale * left(h) + right_scale * right(h) for two split mixers:
     one GEMM projects h for both, each core() writes its head outputs,
@@ -485,7 +696,28 @@ class ParallelMixer(nn.Module):
         return linear(out, self.w_out)
 
 
-def build_mixer(kind: str, m: dict, width: int, eps: float, dtype) -> nn.Module:
+def build_mixer(kind: str, m: dict, width: int, eps: float, dtype,
+                arch: str = "", own_projections: bool = True) -> nn.Module:
+    if arch == "Legalix":
+        if kind == "attention":
+            return SinkRotaryAttention(
+                width, m["heads"], m["kv_heads"], m["dim"], m["vdim"],
+                m["scale"], m["rot"]["base"], m["rot"]["dims"], eps, dtype,
+                qk_norm=False, sink=False, rotate_values=False,
+                interleaved=False, softcap=m["softcap"],
+                window=m["mask"]["size"], keep_first=m["mask"]["keep_first"],
+                own_projections=own_projections)
+        if kind == "latent_attention":
+            return LatentAttention(
+                width, m["heads"], m["dim"], m["rot_dim"], m["vdim"],
+                m["kv_rank"], m["q_rank"], m["scale"], m["rot"]["base"], eps,
+                dtype, own_projections=own_projections)
+        if kind == "mamba2":
+            return Mamba2Mixer(
+                width, m["heads"], m["vdim"], m["state"], m["groups"],
+                m["norm_groups"], m["conv"], eps, dtype,
+                own_projections=own_projections)
+        raise ValueError(f"unknown mixer type {kind!r}")
     if kind == "attention":
         return SinkRotaryAttention(
             width, m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["scale"],

@@ -669,12 +669,38 @@ def sink_attention_tiles(q_lens, kv_lens, num_q_heads, num_kv_heads,
 def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
                          cu_seqlens, token_seq, scale, sink=True,
                          inv_freq_v=None, interleaved=True, max_q_len=0,
-                         positions=None, tiles=None):
+                         positions=None, tiles=None, sink_w=None,
+                         softcap=0.0, window=0, keep_first=0, out=None,
+                         out_scale=1.0):
     """Causal attention of packed rows over paged keys with an optional
-    sink and position-turned values (see ref.attention_sink_paged). bf16
-    rows with equal q/k and value head sizes the MFMA kernels are built for
-    run those (then a pass that turns each row's output back); anything
-    else — float32 rows, other sizes — runs the general kernel."""
+    sink (score 0, or sink_w per head), tanh-capped scores, a sliding
+    window that keeps the first keep_first keys, and position-turned values
+    (see ref.attention_sink_paged). bf16 rows with equal q/k and value head
+    sizes the MFMA kernels are built for run those (then a pass that turns
+    each row's output back); capped, windowed or per-head-sink attention
+    runs the masked matrix-core kernels where they are built; anything else
+    — float32 rows, other sizes — runs the general kernel. out: a [T, H, V]
+    view (rows may be strided) to write, times out_scale."""
+    masked = (sink_w is not None or softcap > 0 or window > 0
+              or out is not None
+              or k_cache.untyped_storage().data_ptr()
+              == v_cache.untyped_storage().data_ptr())
+    if q.is_cuda and masked:
+        T, H, D = q.shape
+        V = v_cache.shape[3]
+        if out is None:
+            out = torch.empty((T, H, V), dtype=q.dtype, device=q.device)
+        S = _native_seq()
+        if not (use_masked_mfma and q.dtype == torch.bfloat16
+                and S.attention_masked_mfma(
+                    out, q, k_cache, v_cache, block_tables, seq_lens,
+                    cu_seqlens, token_seq, scale, sink_w, softcap, window,
+                    keep_first, out_scale, max_q_len == 1)):
+            S.attention_sink_paged(
+                out, q, k_cache, v_cache, block_tables, seq_lens, cu_seqlens,
+                token_seq, scale, sink, None, interleaved, max_q_len, sink_w,
+                softcap, window, keep_first, out_scale)
+        return out
     if q.is_cuda:
         T, H, D = q.shape
         V = v_cache.shape[3]
@@ -702,11 +728,20 @@ def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
         out = torch.empty((T, H, V), dtype=q.dtype, device=q.device)
         _native_seq().attention_sink_paged(
             out, q, k_cache, v_cache, block_tables, seq_lens, cu_seqlens,
-            token_seq, scale, sink, inv_freq_v, interleaved, max_q_len)
+            token_seq, scale, sink, inv_freq_v, interleaved, max_q_len, None,
+            0.0, 0, 0, 1.0)
         return out
-    return ref.attention_sink_paged(q, k_cache, v_cache, block_tables,
-                                    seq_lens, cu_seqlens, scale, sink,
-                                    inv_freq_v, interleaved)
+    res = ref.attention_sink_paged(q, k_cache, v_cache, block_tables,
+                                   seq_lens, cu_seqlens, scale, sink,
+                                   inv_freq_v, interleaved, sink_w, softcap,
+                                   window, keep_first)
+    if out is None:
+        return res
+    out.copy_((res.float() * out_scale).to(out.dtype))
+    return out
+
+
+use_masked_mfma = True  # tests switch it off to compare both paths
 
 
 SCAN_CHUNK = 64  # rows per chunk of the chunk-parallel recurrent prefill
@@ -967,15 +1002,25 @@ def head_norm_gate(o, gate, eps, heads, out, out_scale=1.0):
     return ref.head_norm_gate(o, gate, eps, heads, out, out_scale)
 
 
-def glu_act(gu, kind, limit=0.0, alpha=1.0):
-    """[gate | up] rows -> activated rows (ref.glu_act)."""
+_GLU_MODES = {"swiglu": 0, "clamped": 1, "gelu_tanh": 2}
+
+
+def glu_act(gu, kind, limit=0.0, alpha=1.0, out=None):
+    """[gate | up] rows -> activated rows (ref.glu_act); out: a [T, F]
+    view (rows may be strided) to write instead of a new tensor."""
     if gu.is_cuda:
         F_ = gu.shape[-1] // 2
-        out = torch.empty((gu.shape[0], F_), dtype=gu.dtype, device=gu.device)
-        _native_seq().glu_act(out, gu, 0 if kind == "swiglu" else 1,
-                              float(limit), float(alpha))
+        if out is None:
+            out = torch.empty((gu.shape[0], F_), dtype=gu.dtype,
+                              device=gu.device)
+        _native_seq().glu_act(out, gu, _GLU_MODES[kind], float(limit),
+                              float(alpha))
         return out
-    return ref.glu_act(gu, kind, limit, alpha)
+    res = ref.glu_act(gu, kind, limit, alpha)
+    if out is None:
+        return res
+    out.copy_(res)
+    return out
 
 
 def moe_route_grouped(logits, top, groups, keep):
@@ -1008,3 +1053,87 @@ def moe_mix_rows_seq(y, weights, rows):
         _native_seq().moe_mix_rows(out, y.contiguous(), weights, rows)
         return out
     return ref.moe_mix_rows(y, weights, rows)
+
+
+# ----------------------------------------------------------------------
+# Shared-norm parallel blocks with a tanh norm, latent attention, mamba2
+# (same extension, same rule).
+# ----------------------------------------------------------------------
+def residual_tanh_norm(x, y, mult, alpha, weight, bias, out_dtype, xa=None):
+    """x (fp32 residual, in place) += mult * y when y is given; xa, a
+    [T, C] view of the model's dtype (any row stride), takes the new x;
+    returns tanh(alpha x) * weight + bias in out_dtype (None when weight is
+    None). alpha is a one-element fp32 tensor."""
+    if x.is_cuda:
+        h = (torch.empty(x.shape, dtype=out_dtype, device=x.device)
+             if weight is not None else None)
+        _native_seq().residual_tanh_norm(x, h, xa, y, float(mult), alpha,
+                                         weight, bias)
+        return h
+    return ref.residual_tanh_norm(x, y, mult, alpha, weight, bias, out_dtype, xa)
+
+
+def latent_prepare(cq, ckv, q_norm_w, kv_norm_w, eps, positions, inv_freq,
+                   cache, slot_mapping):
+    """Latent attention's row work before the up-projections
+    (ref.latent_prepare): returns the normed query latent and writes the
+    normed key/value latent with the turned shared key part to its page."""
+    if cq.is_cuda:
+        out = torch.empty(cq.shape, dtype=cq.dtype, device=cq.device)
+        _native_seq().latent_prepare(out, cq, ckv, q_norm_w, kv_norm_w, eps,
+                                     positions, inv_freq, cache, slot_mapping)
+        return out
+    return ref.latent_prepare(cq, ckv, q_norm_w, kv_norm_w, eps, positions,
+                              inv_freq, cache, slot_mapping)
+
+
+def latent_query(q, q_abs, positions, inv_freq, out):
+    """out [T, H, Rk + 2P] = [q_abs ([H, T, Rk]) | turned last 2P dims of q]."""
+    if q.is_cuda:
+        _native_seq().latent_query(out, q, q_abs, positions, inv_freq)
+        return out
+    return ref.latent_query(q, q_abs, positions, inv_freq, out)
+
+
+def mamba2_scan(xbc, dt_raw, dt_bias, rate, Dp, state, cu_seqlens, seq_lens,
+                state_slots, heads, vdim, nstate, groups, max_q_len=0,
+                chunks=None):
+    """Scalar-decay state-space recurrence (ref.mamba2_scan); chunks
+    (scan_chunks of this step): chunk-parallel prefill as lightning_scan —
+    every chunk's end state and summed step sizes from zero state, a
+    combine pass that leaves each chunk's start state, then the outputs."""
+    if xbc.is_cuda:
+        S = _native_seq()
+        T = xbc.shape[0]
+        out = torch.empty((T, heads * vdim), dtype=torch.float32,
+                          device=xbc.device)
+        if chunks is not None and max_q_len > SCAN_CHUNK:
+            c = chunks
+            part = torch.empty((c["n"], heads, nstate, vdim),
+                               dtype=torch.float32, device=xbc.device)
+            dsum = torch.empty((c["n"], heads), dtype=torch.float32,
+                               device=xbc.device)
+            S.mamba2_scan(None, xbc, dt_raw, dt_bias, rate, Dp, part, c["cu"],
+                          c["lens0"], c["slots"], heads, vdim, nstate, groups,
+                          dsum)
+            S.mamba2_combine(part, dsum, rate, state, c["off"], cu_seqlens,
+                             seq_lens, state_slots)
+            S.mamba2_scan(out, xbc, dt_raw, dt_bias, rate, Dp, part, c["cu"],
+                          c["lens1"], c["slots"], heads, vdim, nstate, groups,
+                          None)
+            return out
+        S.mamba2_scan(out, xbc, dt_raw, dt_bias, rate, Dp, state, cu_seqlens,
+                      seq_lens, state_slots, heads, vdim, nstate, groups, None)
+        return out
+    return ref.mamba2_scan(xbc, dt_raw, dt_bias, rate, Dp, state, cu_seqlens,
+                           seq_lens, state_slots, heads, vdim, nstate, groups)
+
+
+def gate_group_norm(y, z, weight, groups, eps, out, out_scale=1.0):
+    """out = per-group unit RMS of (y * silu(z)), times weight and out_scale
+    (ref.gate_group_norm); y fp32, z and out row-strided views."""
+    if y.is_cuda:
+        _native_seq().gate_group_norm(out, y, z, weight, groups, eps,
+                                      out_scale)
+        return out
+    return ref.gate_group_norm(y, z, weight, groups, eps, out, out_scale)

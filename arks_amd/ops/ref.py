@@ -433,11 +433,16 @@ def qk_norm_rope_cache(q, k, v, q_norm_w, k_norm_w, eps, positions,
 
 def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
                          cu_seqlens, scale, sink=True, inv_freq_v=None,
-                         interleaved=True):
+                         interleaved=True, sink_w=None, softcap=0.0,
+                         window=0, keep_first=0):
     """Causal attention of packed new rows over each sequence's paged keys.
     sink=True adds a value-less key of score 0 to every softmax (one more
-    in the denominator). inv_freq_v: each row's output is turned back by its
-    own position over the value dims. q [T,H,D] -> [T,H,V] in q.dtype."""
+    in the denominator); sink_w [H] gives that key a score per head
+    instead (taken as it is: neither scaled nor capped). softcap c > 0:
+    scores become c tanh(score / c). window w > 0: the row at position i
+    sees key j only if i - j < w or j < keep_first. inv_freq_v: each row's
+    output is turned back by its own position over the value dims. v_cache
+    may be a view into k_cache's rows. q [T,H,D] -> [T,H,V] in q.dtype."""
     T, H, D = q.shape
     G, bs, V = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
     out = torch.zeros(T, H, V, dtype=torch.float32)
@@ -457,15 +462,25 @@ def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
         qs = q[a:b].float().permute(1, 0, 2)  # [H, n, D]
         sc = torch.matmul(qs, K.transpose(1, 2)) * scale  # [H, n, L]
         qpos = torch.arange(L - n, L)
-        mask = torch.arange(L)[None, :] > qpos[:, None]
+        if softcap > 0:
+            sc = softcap * torch.tanh(sc / softcap)
+        kpos = torch.arange(L)[None, :]
+        mask = kpos > qpos[:, None]
+        if window > 0:
+            mask = mask | ((qpos[:, None] - kpos >= window)
+                           & (kpos >= keep_first))
         sc = sc.masked_fill(mask[None], float("-inf"))
         m = sc.amax(-1, keepdim=True)
-        if sink:
+        if sink_w is not None:
+            sk = sink_w.float()[:, None, None]
+            m = torch.maximum(m, sk)
+        elif sink:
+            sk = torch.zeros(())
             m = m.clamp(min=0.0)
         e = torch.exp(sc - m)
         den = e.sum(-1, keepdim=True)
-        if sink:
-            den = den + torch.exp(-m)
+        if sink or sink_w is not None:
+            den = den + torch.exp(sk - m)
         o = torch.matmul(e / den, Vv).permute(1, 0, 2)  # [n, H, V]
         if inv_freq_v is not None:
             ang = -qpos.float()[:, None, None] * inv_freq_v.float()[None, None, :]
@@ -736,11 +751,14 @@ def glu_act(gu, kind, limit=0.0, alpha=1.0):
     """gu [T, 2F] = [gate | up] -> [T, F].
     "swiglu": silu(gate) * up.
     "clamped": g = min(gate, limit), u = clamp(up, -limit, limit),
-               g * sigmoid(alpha g) * (u + 1)."""
+               g * sigmoid(alpha g) * (u + 1).
+    "gelu_tanh": gelu_tanh(gate) * up."""
     F_ = gu.shape[-1] // 2
     g, u = gu[..., :F_].float(), gu[..., F_:].float()
     if kind == "swiglu":
         return (g * torch.sigmoid(g) * u).to(gu.dtype)
+    if kind == "gelu_tanh":
+        return (torch.nn.functional.gelu(g, approximate="tanh") * u).to(gu.dtype)
     g = g.clamp(max=limit)
     u = u.clamp(-limit, limit)
     return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
@@ -765,3 +783,96 @@ def moe_route_grouped(logits, top, groups, keep):
     w = s.gather(1, ids)
     w = w / (w.sum(-1, keepdim=True) + 1e-20)
     return w, ids.to(torch.int32)
+
+
+# ----------------------------------------------------------------------
+# Shared-norm parallel blocks with a tanh norm, latent attention, mamba2.
+# ----------------------------------------------------------------------
+def residual_tanh_norm(x, y, mult, alpha, weight, bias, out_dtype, xa=None):
+    """x (fp32, in place) += mult * y when y is given; xa (a [T, C] view,
+    any row stride) takes the new x in its own dtype; returns
+    tanh(alpha x) * weight + bias in out_dtype (None without a weight)."""
+    if y is not None:
+        x += mult * y.float()
+    if xa is not None:
+        xa.copy_(x)
+    if weight is None:
+        return None
+    return (torch.tanh(alpha.float() * x) * weight.float()
+            + bias.float()).to(out_dtype)
+
+
+def latent_prepare(cq, ckv, q_norm_w, kv_norm_w, eps, positions, inv_freq,
+                   cache, slot_mapping):
+    """Row work of latent attention before its up-projections. cq [T, Rq]:
+    RMS norm times q_norm_w, returned in cq.dtype. ckv [T, Rk + 2P]: the
+    first Rk columns RMS-normed times kv_norm_w, the last 2P (P =
+    len(inv_freq)) turned by the row's position in interleaved pairs; the
+    row goes to its place in cache [blocks, 1, bs, Rk + 2P]."""
+    def unit(t):
+        return t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps)
+
+    cqn = (unit(cq.float()) * q_norm_w.float()).to(cq.dtype)
+    rank = kv_norm_w.shape[0]
+    f = ckv.float()
+    c = unit(f[:, :rank]) * kv_norm_w.float()
+    ang = positions.float()[:, None] * inv_freq.float()[None, :]
+    kr = _rotate_pairs(f[:, rank:], ang, True)
+    row = torch.cat([c, kr], -1).to(cache.dtype)
+    bs = cache.shape[2]
+    ok = slot_mapping >= 0
+    cache[(slot_mapping[ok] // bs).long(), 0, (slot_mapping[ok] % bs).long()] = row[ok]
+    return cqn
+
+
+def latent_query(q, q_abs, positions, inv_freq, out):
+    """out [T, H, Rk + 2P] = [q_abs (given as [H, T, Rk]) | the last 2P
+    dims of q [T, H, D + 2P] turned by the row's position, interleaved]."""
+    rank = q_abs.shape[2]
+    D = q.shape[2] - 2 * inv_freq.numel()
+    ang = positions.float()[:, None, None] * inv_freq.float()[None, None, :]
+    out[..., :rank] = q_abs.transpose(0, 1)
+    out[..., rank:] = _rotate_pairs(q[..., D:].float(), ang, True).to(out.dtype)
+    return out
+
+
+def mamba2_scan(xbc, dt_raw, dt_bias, rate, Dp, state, cu_seqlens, seq_lens,
+                state_slots, heads, vdim, nstate, groups):
+    """Scalar-decay state-space recurrence per head: xbc [T, P*V + 2*G*N] =
+    [x | B | C] (after conv and silu), dt = softplus(dt_raw + dt_bias) [T, P];
+    S_h (N x V) <- exp(-rate_h dt) S_h + dt B_g x_h^T,
+    y_h = S_h^T C_g + D_h x_h with g = h // (P / G). state
+    [slots, P, N, V] fp32 (updated). Returns y fp32 [T, P*V]."""
+    T = xbc.shape[0]
+    P, V, N, G = heads, vdim, nstate, groups
+    f = xbc.float()
+    x = f[:, :P * V].reshape(T, P, V)
+    Bm = f[:, P * V:P * V + G * N].reshape(T, G, N).repeat_interleave(P // G, 1)
+    Cm = f[:, P * V + G * N:].reshape(T, G, N).repeat_interleave(P // G, 1)
+    dt = torch.nn.functional.softplus(dt_raw.float() + dt_bias.float(),
+                                      threshold=20.0)
+    a = torch.exp(-rate.float()[None, :] * dt)  # [T, P]
+    out = torch.empty(T, P, V, dtype=torch.float32)
+    for lo, hi, start, slot in _seq_spans(cu_seqlens, seq_lens, state_slots):
+        S = (state[slot].clone() if start > 0 and slot >= 0
+             else torch.zeros(P, N, V))
+        for t in range(lo, hi):
+            S = a[t][:, None, None] * S + \
+                (dt[t][:, None] * Bm[t])[:, :, None] * x[t][:, None, :]
+            out[t] = torch.einsum("pnv,pn->pv", S, Cm[t]) \
+                + Dp.float()[:, None] * x[t]
+        if slot >= 0:
+            state[slot] = S
+    return out.reshape(T, P * V)
+
+
+def gate_group_norm(y, z, weight, groups, eps, out, out_scale=1.0):
+    """out = unit_rms_per_group(y * silu(z)) * weight * out_scale: the row
+    is cut into `groups` equal parts, each divided by its own root mean
+    square. y fp32 [T, C]; z, out [T, C] views."""
+    T, C = y.shape
+    g = y.float() * torch.nn.functional.silu(z.float())
+    g = g.view(T, groups, C // groups)
+    g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)
+    out.copy_((g.reshape(T, C) * weight.float() * out_scale).to(out.dtype))
+    return out
