@@ -52,6 +52,9 @@ SEQ_SOURCES = [
     os.path.join(CSRC, "seq_window.hip"),
     os.path.join(CSRC, "seq_window_mfma.hip"),
     os.path.join(CSRC, "seq_moe.hip"),
+    os.path.join(CSRC, "seq_shared.hip"),
+    os.path.join(CSRC, "seq_mamba2.hip"),
+    os.path.join(CSRC, "seq_masked_mfma.hip"),
 ]
 
 EXTENSIONS = {EXT_NAME: SOURCES, SEQ_EXT_NAME: SEQ_SOURCES}

@@ -8,14 +8,20 @@
 // the running maximum and rescales, then every lane accumulates its own
 // value dims over the tile's 64 weights. The softmax may carry a sink: a
 // key of score 0 without a value, i.e. the running state starts at
-// (max 0, sum 1) instead of (-inf, 0). After the sum each row's output is
-// turned back by its own position when the cache holds position-turned
-// values.
+// (max 0, sum 1) instead of (-inf, 0); with sink_w the sink's score is a
+// number per head, (max sink_w[h], sum 1). softcap c > 0 turns a score s
+// into c tanh(s / c). window w > 0: the row at position i sees key j <= i
+// only if i - j < w or j < keep_first; tiles with no visible key are
+// skipped. Key and value rows have their own strides (ldk, ldv), so the
+// value may be a leading part of the key's row (latent attention keeps one
+// row per token for both). The output is a row-strided view (ldo), scaled
+// by out_scale. After the sum each row's output is turned back by its own
+// position when the cache holds position-turned values.
 #include "seq_common.h"
 
 namespace arks {
 
-constexpr int ATT_MAX_D = 512;  // query dims held in LDS
+constexpr int ATT_MAX_D = 1024;  // query dims held in LDS
 constexpr int ATT_VPT = 8;      // value dims per lane (V <= 512)
 
 template <typename AT>
@@ -25,7 +31,9 @@ __global__ __launch_bounds__(64) void attn_sink_generic_kernel(
     const int* __restrict__ block_tables, const int* __restrict__ seq_lens,
     const int* __restrict__ cu, const int* __restrict__ token_seq,
     float scale, int sink, const float* __restrict__ freq_v, int interleaved,
-    int H, int G, int D, int V, int block_size, int max_blocks) {
+    int H, int G, int D, int V, int block_size, int max_blocks,
+    const float* __restrict__ sink_w, float softcap, int window,
+    int keep_first, int64_t ldk, int64_t ldv, int64_t ldo, float out_scale) {
   __shared__ float q_s[ATT_MAX_D];
   __shared__ float p_s[64];
   __shared__ int64_t voff_s[64];
@@ -41,23 +49,27 @@ __global__ __launch_bounds__(64) void attn_sink_generic_kernel(
   for (int d = lane; d < D; d += 64)
     q_s[d] = Act<AT>::ld(q + ((int64_t)t * H + h) * D + d);
   __syncthreads();
-  float m = sink ? 0.f : -INFINITY;
-  float l = sink ? 1.f : 0.f;
+  float m = sink_w ? sink_w[h] : (sink ? 0.f : -INFINITY);
+  float l = (sink_w || sink) ? 1.f : 0.f;
   float acc[ATT_VPT];
 #pragma unroll
   for (int i = 0; i < ATT_VPT; ++i) acc[i] = 0.f;
+  // first key of the window; keys in [keep_first, lo) are hidden
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   for (int j0 = 0; j0 < nkeys; j0 += 64) {
+    if (j0 >= keep_first && j0 + 64 <= lo) continue;
     const int j = j0 + lane;
-    const bool valid = j < nkeys;
+    const bool valid = j < nkeys && (j >= lo || j < keep_first);
     float sc = -INFINITY;
     int64_t rowoff = 0;
     if (valid) {
       const int page = bt[j / block_size];
       rowoff = ((int64_t)page * G + g) * block_size + (j % block_size);
-      const AT* kr = k_cache + rowoff * D;
+      const AT* kr = k_cache + rowoff * ldk;
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot += q_s[d] * Act<AT>::ld(kr + d);
       sc = dot * scale;
+      if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
     }
     const float m_new = fmaxf(m, wave_reduce_max(sc));
     const float p = valid ? expf(sc - m_new) : 0.f;
@@ -68,11 +80,12 @@ __global__ __launch_bounds__(64) void attn_sink_generic_kernel(
     m = m_new;
     __syncthreads();  // previous tile's readers are done
     p_s[lane] = p;
-    voff_s[lane] = rowoff * V;
+    voff_s[lane] = rowoff * ldv;
     __syncthreads();
     const int cnt = min(64, nkeys - j0);
     for (int jj = 0; jj < cnt; ++jj) {
       const float pj = p_s[jj];
+      if (pj == 0.f) continue;  // hidden key (uniform over the wave)
       const AT* vr = v_cache + voff_s[jj];
 #pragma unroll
       for (int i = 0; i < ATT_VPT; ++i) {
@@ -81,8 +94,8 @@ __global__ __launch_bounds__(64) void attn_sink_generic_kernel(
       }
     }
   }
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  AT* orow = out + ((int64_t)t * H + h) * V;
+  const float inv = l > 0.f ? out_scale / l : 0.f;
+  AT* orow = out + (int64_t)t * ldo + (int64_t)h * V;
   if (!freq_v) {
 #pragma unroll
     for (int i = 0; i < ATT_VPT; ++i) {
@@ -119,7 +132,9 @@ extern "C" int arks_seq_attn_sink_generic(
     const void* block_tables, const void* seq_lens, const void* cu,
     const void* token_seq, float scale, int sink, const void* freq_v,
     int interleaved, int T, int H, int G, int D, int V, int block_size,
-    int max_blocks, int act_f32, hipStream_t stream) {
+    int max_blocks, int act_f32, const void* sink_w, float softcap,
+    int window, int keep_first, int64_t ldk, int64_t ldv, int64_t ldo,
+    float out_scale, hipStream_t stream) {
   if (D > ATT_MAX_D || V > 64 * ATT_VPT) return 1;
   if (T == 0) return 0;
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
@@ -127,6 +142,7 @@ extern "C" int arks_seq_attn_sink_generic(
       (AT*)out, (const AT*)q, (const AT*)k_cache, (const AT*)v_cache,
       (const int*)block_tables, (const int*)seq_lens, (const int*)cu,
       (const int*)token_seq, scale, sink, (const float*)freq_v, interleaved, H,
-      G, D, V, block_size, max_blocks));
+      G, D, V, block_size, max_blocks, (const float*)sink_w, softcap, window,
+      keep_first, ldk, ldv, ldo, out_scale));
   return 0;
 }

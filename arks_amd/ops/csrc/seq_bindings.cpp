@@ -36,7 +36,9 @@ int arks_seq_attn_sink_generic(
     const void* block_tables, const void* seq_lens, const void* cu,
     const void* token_seq, float scale, int sink, const void* freq_v,
     int interleaved, int T, int H, int G, int D, int V, int block_size,
-    int max_blocks, int act_f32, hipStream_t stream);
+    int max_blocks, int act_f32, const void* sink_w, float softcap,
+    int window, int keep_first, int64_t ldk, int64_t ldv, int64_t ldo,
+    float out_scale, hipStream_t stream);
 int arks_seq_lightning_scan(void* out, const void* q, const void* k,
                             const void* v, int64_t ldq, int64_t ldk,
                             int64_t ldv, const void* decay, void* state,
@@ -85,9 +87,9 @@ void arks_seq_head_norm_gate(void* out, int64_t ldo, const void* o,
                              const void* gate, int64_t ldg, float eps, int T,
                              int H, int V, float out_scale, int act_f32,
                              hipStream_t stream);
-void arks_seq_glu_act(void* out, const void* gu, int64_t ldg, int64_t rows,
-                      int F, int mode, float limit, float alpha, int act_f32,
-                      hipStream_t stream);
+void arks_seq_glu_act(void* out, int64_t ldo, const void* gu, int64_t ldg,
+                      int64_t rows, int F, int mode, float limit, float alpha,
+                      int act_f32, hipStream_t stream);
 void arks_seq_kv_write_pooled(const void* k, const void* v, int64_t ldk,
                               int64_t ldv, void* k_cache, void* v_cache,
                               void* kp_cache, void* vp_cache,
@@ -117,6 +119,46 @@ int arks_seq_attn_window_pool_mfma(void* out, int64_t ldo, const void* q,
                                    int V, int bs, int max_blocks,
                                    int num_seqs, int single_rows,
                                    hipStream_t stream);
+void arks_seq_residual_tanh_norm(void* x, void* h, void* xa, int64_t ldxa,
+                                 const void* y, float mult, const void* alpha,
+                                 const void* w, const void* b, int64_t T, int C,
+                                 int act_f32, hipStream_t stream);
+void arks_seq_latent_prepare(void* cqn, const void* cq, int64_t ldq,
+                             const void* ckv, int64_t ldk, const void* qw,
+                             const void* kw, float eps, const void* positions,
+                             const void* freq, void* cache,
+                             const void* slot_mapping, int T, int Rq, int Rk,
+                             int P, int act_f32, hipStream_t stream);
+void arks_seq_latent_query(void* out, const void* q, const void* q_abs,
+                           const void* positions, const void* freq, int T,
+                           int H, int D, int Rk, int P, int act_f32,
+                           hipStream_t stream);
+int arks_seq_mamba2_scan(void* out, const void* xbc, int64_t ldx,
+                         const void* dt_raw, int64_t ldd, const void* dt_bias,
+                         const void* rate, const void* Dp, void* state,
+                         const void* cu, const void* seq_lens,
+                         const void* slots, void* dsum, int S, int P, int V,
+                         int N, int G, int act_f32, hipStream_t stream);
+void arks_seq_mamba2_combine(void* part, const void* dsum, const void* rate,
+                             void* state, const void* chunk_off,
+                             const void* cu, const void* seq_lens,
+                             const void* slots, int S, int P, int NV,
+                             hipStream_t stream);
+void arks_seq_gate_group_norm(void* out, int64_t ldo, const void* y,
+                              const void* z, int64_t ldz, const void* w,
+                              float eps, int T, int C, int groups,
+                              float out_scale, int act_f32,
+                              hipStream_t stream);
+int arks_seq_attn_masked_mfma(void* out, int64_t ldo, const void* q,
+                              const void* k_cache, int64_t ldk,
+                              const void* v_cache, int64_t ldv,
+                              const void* block_tables, const void* seq_lens,
+                              const void* cu, const void* token_seq,
+                              float scale, const void* sink_w, float softcap,
+                              int window, int keep_first, float out_scale,
+                              int T, int H, int G, int D, int V, int bs,
+                              int max_blocks, int num_seqs, int single_rows,
+                              hipStream_t stream);
 int arks_seq_moe_route_grouped(void* weights, void* ids, const void* logits,
                                int T, int E, int top, int groups, int keep,
                                hipStream_t stream);
@@ -177,6 +219,17 @@ int64_t head_row_stride(const Tensor& t, const char* name) {
   TORCH_CHECK(t.dim() == 3 && t.stride(2) == 1 && t.stride(1) == t.size(2),
               name, " must be [T, heads, dim] with dense heads");
   return t.stride(0);
+}
+
+// [pages, G, bs, dim] cache, or a view of the leading columns of one:
+// token rows a fixed stride apart through heads and pages; returns it
+int64_t paged_row_stride(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.dim() == 4 && t.stride(3) == 1 &&
+                  t.stride(1) == t.size(2) * t.stride(2) &&
+                  t.stride(0) == t.size(1) * t.stride(1) &&
+                  t.stride(2) >= t.size(3),
+              name, " must be [pages, heads, tokens, dim] rows of one stride");
+  return t.stride(2);
 }
 
 struct SeqMeta {
@@ -346,19 +399,29 @@ void attention_sink_paged(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
                           Tensor block_tables, Tensor seq_lens, Tensor cu,
                           Tensor token_seq, double scale, bool sink,
                           OptTensor freq_v, bool interleaved,
-                          int64_t max_q_len) {
+                          int64_t max_q_len, OptTensor sink_w, double softcap,
+                          int64_t window, int64_t keep_first,
+                          double out_scale) {
   const int f32 = act_flag(q, "q");
   TORCH_CHECK(q.is_contiguous() && q.dim() == 3);
   const int T = q.size(0), H = q.size(1), D = q.size(2);
   TORCH_CHECK(k_cache.scalar_type() == q.scalar_type() &&
               v_cache.scalar_type() == q.scalar_type() &&
               out.scalar_type() == q.scalar_type());
-  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
-              k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(3) == D);
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(3) == D);
   const int G = k_cache.size(1), bs = k_cache.size(2), V = v_cache.size(3);
   TORCH_CHECK(H % G == 0 && v_cache.size(1) == G && v_cache.size(2) == bs);
-  TORCH_CHECK(out.is_contiguous() && out.size(0) == T && out.size(1) == H &&
-              out.size(2) == V);
+  const int64_t ldk = paged_row_stride(k_cache, "k_cache");
+  const int64_t ldv = paged_row_stride(v_cache, "v_cache");
+  const int64_t ldo = head_row_stride(out, "out");
+  TORCH_CHECK(out.size(0) == T && out.size(1) == H && out.size(2) == V);
+  const void* sw_p = nullptr;
+  if (sink_w.has_value()) {
+    check_f32(*sink_w, "sink_w");
+    TORCH_CHECK(sink_w->numel() == H);
+    sw_p = sink_w->data_ptr();
+  }
+  TORCH_CHECK(window >= 0 && keep_first >= 0 && softcap >= 0);
   check_i32(block_tables, "block_tables");
   TORCH_CHECK(block_tables.dim() == 2 &&
               block_tables.size(0) == seq_lens.numel());
@@ -374,7 +437,8 @@ void attention_sink_paged(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
       block_tables.data_ptr(), seq_lens.data_ptr(), cu.data_ptr(),
       token_seq.data_ptr(), (float)scale, sink ? 1 : 0, fv_p,
       interleaved ? 1 : 0, T, H, G, D, V, bs, (int)block_tables.size(1), f32,
-      current_stream());
+      sw_p, (float)softcap, (int)window, (int)keep_first, ldk, ldv, ldo,
+      (float)out_scale, current_stream());
   TORCH_CHECK(rc == 0, "attention head sizes beyond the kernel's limits (",
               D, ", ", V, ")");
 }
@@ -699,11 +763,11 @@ void glu_act(Tensor out, Tensor gu, int64_t mode, double limit, double alpha) {
   const int f32 = act_flag(gu, "gate|up");
   TORCH_CHECK(gu.dim() == 2 && gu.size(1) % 2 == 0);
   const int F = gu.size(1) / 2;
-  TORCH_CHECK(out.scalar_type() == gu.scalar_type() && out.is_contiguous() &&
+  TORCH_CHECK(out.scalar_type() == gu.scalar_type() &&
               out.size(0) == gu.size(0) && out.size(1) == F);
-  arks_seq_glu_act(out.data_ptr(), gu.data_ptr(), row_stride(gu, "gate|up"),
-                   gu.size(0), F, (int)mode, (float)limit, (float)alpha, f32,
-                   current_stream());
+  arks_seq_glu_act(out.data_ptr(), row_stride(out, "out"), gu.data_ptr(),
+                   row_stride(gu, "gate|up"), gu.size(0), F, (int)mode,
+                   (float)limit, (float)alpha, f32, current_stream());
 }
 
 struct WindowShapes {
@@ -858,7 +922,224 @@ void moe_mix_rows(Tensor out, Tensor y, Tensor weights, Tensor rows) {
 
 }  // namespace
 
+void residual_tanh_norm(Tensor x, OptTensor h, OptTensor xa, OptTensor y,
+                        double mult, OptTensor alpha, OptTensor w,
+                        OptTensor b) {
+  check_f32(x, "x");
+  TORCH_CHECK(x.dim() == 2);
+  const int64_t T = x.size(0);
+  const int C = x.size(1);
+  int f32 = -1;
+  auto same = [&](const Tensor& t, const char* name) {
+    const int f = act_flag(t, name);
+    TORCH_CHECK(f32 < 0 || f == f32, "activation dtypes differ");
+    f32 = f;
+    TORCH_CHECK(t.dim() == 2 && t.size(0) == T && t.size(1) == C, name,
+                " must be [T, C]");
+  };
+  void* h_p = nullptr;
+  void* xa_p = nullptr;
+  const void* y_p = nullptr;
+  int64_t ldxa = C;
+  if (h.has_value()) {
+    same(*h, "h");
+    TORCH_CHECK(h->is_contiguous() && alpha.has_value() && w.has_value() &&
+                b.has_value());
+    check_f32(*alpha, "alpha");
+    check_f32(*w, "weight");
+    check_f32(*b, "bias");
+    TORCH_CHECK(alpha->numel() == 1 && w->numel() == C && b->numel() == C);
+    h_p = h->data_ptr();
+  }
+  if (xa.has_value()) {
+    same(*xa, "xa");
+    ldxa = row_stride(*xa, "xa");
+    xa_p = xa->data_ptr();
+  }
+  if (y.has_value()) {
+    same(*y, "y");
+    TORCH_CHECK(y->is_contiguous());
+    y_p = y->data_ptr();
+  }
+  if (f32 < 0) return;  // nothing to add, nothing to write
+  arks_seq_residual_tanh_norm(
+      x.data_ptr(), h_p, xa_p, ldxa, y_p, (float)mult,
+      alpha.has_value() ? alpha->data_ptr() : nullptr,
+      w.has_value() ? w->data_ptr() : nullptr,
+      b.has_value() ? b->data_ptr() : nullptr, T, C, f32, current_stream());
+}
+
+void latent_prepare(Tensor cqn, Tensor cq, Tensor ckv, Tensor qw, Tensor kw,
+                    double eps, Tensor positions, Tensor freq, Tensor cache,
+                    Tensor slot_mapping) {
+  const int f32 = act_flag(cq, "cq");
+  const int T = cq.size(0), Rq = cq.size(1);
+  check_f32(qw, "q norm");
+  check_f32(kw, "kv norm");
+  check_f32(freq, "inv_freq");
+  const int Rk = kw.numel(), P = freq.numel();
+  TORCH_CHECK(cqn.scalar_type() == cq.scalar_type() && cqn.is_contiguous() &&
+              cqn.size(0) == T && cqn.size(1) == Rq && qw.numel() == Rq);
+  TORCH_CHECK(ckv.scalar_type() == cq.scalar_type() && ckv.dim() == 2 &&
+              ckv.size(0) == T && ckv.size(1) == Rk + 2 * P);
+  TORCH_CHECK(cache.scalar_type() == cq.scalar_type() && cache.is_contiguous() &&
+              cache.dim() == 4 && cache.size(1) == 1 &&
+              cache.size(3) == Rk + 2 * P);
+  check_i64(positions, "positions");
+  check_i64(slot_mapping, "slot_mapping");
+  TORCH_CHECK(positions.numel() == T && slot_mapping.numel() == T);
+  arks_seq_latent_prepare(cqn.data_ptr(), cq.data_ptr(), row_stride(cq, "cq"),
+                          ckv.data_ptr(), row_stride(ckv, "ckv"), qw.data_ptr(),
+                          kw.data_ptr(), (float)eps, positions.data_ptr(),
+                          freq.data_ptr(), cache.data_ptr(),
+                          slot_mapping.data_ptr(), T, Rq, Rk, P, f32,
+                          current_stream());
+}
+
+void latent_query(Tensor out, Tensor q, Tensor q_abs, Tensor positions,
+                  Tensor freq) {
+  const int f32 = act_flag(q, "q");
+  check_f32(freq, "inv_freq");
+  check_i64(positions, "positions");
+  TORCH_CHECK(q.dim() == 3 && q.is_contiguous() && q_abs.dim() == 3 &&
+              q_abs.is_contiguous() && out.dim() == 3 && out.is_contiguous());
+  const int T = q.size(0), H = q.size(1), P = freq.numel();
+  const int D = q.size(2) - 2 * P, Rk = q_abs.size(2);
+  TORCH_CHECK(D >= 0 && q_abs.size(0) == H && q_abs.size(1) == T &&
+              out.size(0) == T && out.size(1) == H &&
+              out.size(2) == Rk + 2 * P && positions.numel() == T &&
+              q_abs.scalar_type() == q.scalar_type() &&
+              out.scalar_type() == q.scalar_type());
+  arks_seq_latent_query(out.data_ptr(), q.data_ptr(), q_abs.data_ptr(),
+                        positions.data_ptr(), freq.data_ptr(), T, H, D, Rk, P,
+                        f32, current_stream());
+}
+
+void mamba2_scan(OptTensor out, Tensor xbc, Tensor dt_raw, Tensor dt_bias,
+                 Tensor rate, Tensor Dp, Tensor state, Tensor cu,
+                 Tensor seq_lens, Tensor slots, int64_t P, int64_t V,
+                 int64_t N, int64_t G, OptTensor dsum) {
+  const int f32 = act_flag(xbc, "xbc");
+  const int64_t T = xbc.size(0);
+  TORCH_CHECK(dt_raw.scalar_type() == xbc.scalar_type() && dt_raw.dim() == 2 &&
+              dt_raw.size(0) == T && dt_raw.size(1) == P);
+  TORCH_CHECK(xbc.dim() == 2 && xbc.size(1) == P * V + 2 * G * N && G >= 1 &&
+              P % G == 0);
+  check_f32(dt_bias, "dt_bias");
+  check_f32(rate, "rate");
+  check_f32(Dp, "D");
+  check_f32(state, "state");
+  TORCH_CHECK(dt_bias.numel() == P && rate.numel() == P && Dp.numel() == P);
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == P && state.size(2) == N &&
+              state.size(3) == V);
+  const SeqMeta m = check_meta(cu, seq_lens, &slots, nullptr, 0);
+  void* out_p = nullptr;
+  if (out.has_value()) {
+    check_f32(*out, "out");
+    TORCH_CHECK(out->dim() == 2 && out->size(0) == T && out->size(1) == P * V);
+    out_p = out->data_ptr();
+  }
+  void* ds_p = nullptr;
+  if (dsum.has_value()) {
+    check_f32(*dsum, "dsum");
+    TORCH_CHECK(dsum->dim() == 2 && dsum->size(0) == state.size(0) &&
+                dsum->size(1) == P);
+    ds_p = dsum->data_ptr();
+  }
+  const int rc = arks_seq_mamba2_scan(
+      out_p, xbc.data_ptr(), row_stride(xbc, "xbc"), dt_raw.data_ptr(),
+      row_stride(dt_raw, "dt"), dt_bias.data_ptr(), rate.data_ptr(),
+      Dp.data_ptr(), state.data_ptr(), cu.data_ptr(), seq_lens.data_ptr(),
+      slots.data_ptr(), ds_p, m.S, (int)P, (int)V, (int)N, (int)G, f32,
+      current_stream());
+  TORCH_CHECK(rc == 0, "mamba2 state size beyond the kernel's limit (", N, ")");
+}
+
+void mamba2_combine(Tensor part, Tensor dsum, Tensor rate, Tensor state,
+                    Tensor chunk_off, Tensor cu, Tensor seq_lens,
+                    Tensor slots) {
+  check_f32(part, "part");
+  check_f32(dsum, "dsum");
+  check_f32(rate, "rate");
+  check_f32(state, "state");
+  const int P = rate.numel();
+  TORCH_CHECK(part.dim() == 4 && state.dim() == 4 && part.size(1) == P &&
+              state.size(1) == P && part.size(2) == state.size(2) &&
+              part.size(3) == state.size(3) && dsum.dim() == 2 &&
+              dsum.size(0) == part.size(0) && dsum.size(1) == P);
+  const SeqMeta m = check_meta(cu, seq_lens, &slots, nullptr, 0);
+  check_i32(chunk_off, "chunk_off");
+  TORCH_CHECK(chunk_off.numel() == m.S + 1);
+  arks_seq_mamba2_combine(part.data_ptr(), dsum.data_ptr(), rate.data_ptr(),
+                          state.data_ptr(), chunk_off.data_ptr(), cu.data_ptr(),
+                          seq_lens.data_ptr(), slots.data_ptr(), m.S, P,
+                          (int)(part.size(2) * part.size(3)), current_stream());
+}
+
+void gate_group_norm(Tensor out, Tensor y, Tensor z, Tensor w, int64_t groups,
+                     double eps, double out_scale) {
+  check_f32(y, "y");
+  check_f32(w, "weight");
+  const int f32 = act_flag(z, "z");
+  TORCH_CHECK(y.dim() == 2);
+  const int T = y.size(0), C = y.size(1);
+  TORCH_CHECK(groups >= 1 && C % groups == 0 && w.numel() == C);
+  TORCH_CHECK(out.scalar_type() == z.scalar_type() && z.dim() == 2 &&
+              z.size(0) == T && z.size(1) == C && out.dim() == 2 &&
+              out.size(0) == T && out.size(1) == C);
+  arks_seq_gate_group_norm(out.data_ptr(), row_stride(out, "out"), y.data_ptr(),
+                           z.data_ptr(), row_stride(z, "z"), w.data_ptr(),
+                           (float)eps, T, C, (int)groups, (float)out_scale, f32,
+                           current_stream());
+}
+
+// false: no matrix-core kernel for these sizes (the caller runs the general
+// one)
+bool attention_masked_mfma(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
+                           Tensor block_tables, Tensor seq_lens, Tensor cu,
+                           Tensor token_seq, double scale, OptTensor sink_w,
+                           double softcap, int64_t window, int64_t keep_first,
+                           double out_scale, bool single_rows) {
+  TORCH_CHECK(q.is_cuda() && q.scalar_type() == torch::kBFloat16 &&
+              q.is_contiguous() && q.dim() == 3);
+  const int T = q.size(0), H = q.size(1), D = q.size(2);
+  TORCH_CHECK(k_cache.scalar_type() == q.scalar_type() &&
+              v_cache.scalar_type() == q.scalar_type() &&
+              out.scalar_type() == q.scalar_type());
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(3) == D);
+  const int G = k_cache.size(1), bs = k_cache.size(2), V = v_cache.size(3);
+  TORCH_CHECK(H % G == 0 && v_cache.size(1) == G && v_cache.size(2) == bs);
+  const int64_t ldk = paged_row_stride(k_cache, "k_cache");
+  const int64_t ldv = paged_row_stride(v_cache, "v_cache");
+  const int64_t ldo = head_row_stride(out, "out");
+  TORCH_CHECK(out.size(0) == T && out.size(1) == H && out.size(2) == V);
+  const void* sw_p = nullptr;
+  if (sink_w.has_value()) {
+    check_f32(*sink_w, "sink_w");
+    TORCH_CHECK(sink_w->numel() == H);
+    sw_p = sink_w->data_ptr();
+  }
+  check_i32(block_tables, "block_tables");
+  TORCH_CHECK(block_tables.dim() == 2 &&
+              block_tables.size(0) == seq_lens.numel());
+  const SeqMeta m = check_meta(cu, seq_lens, nullptr, &token_seq, T);
+  return arks_seq_attn_masked_mfma(
+             out.data_ptr(), ldo, q.data_ptr(), k_cache.data_ptr(), ldk,
+             v_cache.data_ptr(), ldv, block_tables.data_ptr(),
+             seq_lens.data_ptr(), cu.data_ptr(), token_seq.data_ptr(),
+             (float)scale, sw_p, (float)softcap, (int)window, (int)keep_first,
+             (float)out_scale, T, H, G, D, V, bs, (int)block_tables.size(1),
+             m.S, single_rows ? 1 : 0, current_stream()) == 0;
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("residual_tanh_norm", &residual_tanh_norm);
+  m.def("latent_prepare", &latent_prepare);
+  m.def("latent_query", &latent_query);
+  m.def("mamba2_scan", &mamba2_scan);
+  m.def("mamba2_combine", &mamba2_combine);
+  m.def("gate_group_norm", &gate_group_norm);
+  m.def("attention_masked_mfma", &attention_masked_mfma);
   m.def("stream_mix_norm", &stream_mix_norm);
   m.def("short_conv_residual", &short_conv_residual);
   m.def("head_norm_gate", &head_norm_gate);

@@ -352,32 +352,37 @@ __global__ __launch_bounds__(64) void head_norm_gate_kernel(
 }
 
 // mode 0: silu(g) * u;  mode 1: g = min(g, limit), u = clamp(u, +-limit),
-// g * sigmoid(alpha g) * (u + 1)
+// g * sigmoid(alpha g) * (u + 1);  mode 2: gelu_tanh(g) * u. The output is
+// a row-strided view (ldo).
+__device__ __forceinline__ float glu_value(float g, float u, int mode,
+                                           float limit, float alpha) {
+  if (mode == 0) return silu_f(g) * u;
+  if (mode == 2) {
+    const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    return 0.5f * g * (1.f + tanhf(z)) * u;
+  }
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g * sigmoid_f(alpha * g) * (u + 1.f);
+}
+
 template <typename AT>
 __global__ __launch_bounds__(256) void glu_act_kernel(
-    AT* __restrict__ out, const AT* __restrict__ gu, int64_t ldg, int64_t rows,
-    int F, int mode, float limit, float alpha) {
+    AT* __restrict__ out, int64_t ldo, const AT* __restrict__ gu, int64_t ldg,
+    int64_t rows, int F, int mode, float limit, float alpha) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= rows * F) return;
   const int64_t t = i / F;
   const int c = (int)(i - t * F);
-  float g = Act<AT>::ld(gu + t * ldg + c);
-  float u = Act<AT>::ld(gu + t * ldg + F + c);
-  float r;
-  if (mode == 0) {
-    r = silu_f(g) * u;
-  } else {
-    g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit);
-    r = g * sigmoid_f(alpha * g) * (u + 1.f);
-  }
-  Act<AT>::st(out + i, r);
+  const float g = Act<AT>::ld(gu + t * ldg + c);
+  const float u = Act<AT>::ld(gu + t * ldg + F + c);
+  Act<AT>::st(out + t * ldo + c, glu_value(g, u, mode, limit, alpha));
 }
 
 // bf16, 8 elements per thread (F % 8 == 0, 16-byte aligned rows)
 __global__ __launch_bounds__(256) void glu_act_vec8_kernel(
-    bf16* __restrict__ out, const bf16* __restrict__ gu, int64_t ldg,
-    int64_t rows, int F, int mode, float limit, float alpha) {
+    bf16* __restrict__ out, int64_t ldo, const bf16* __restrict__ gu,
+    int64_t ldg, int64_t rows, int F, int mode, float limit, float alpha) {
   const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
   if (i >= rows * F) return;
   const int64_t t = i / F;
@@ -387,17 +392,11 @@ __global__ __launch_bounds__(256) void glu_act_vec8_kernel(
   ushort8 o;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    float g = bf16_bits_to_float(gv[e]), u = bf16_bits_to_float(uv[e]), r;
-    if (mode == 0) {
-      r = silu_f(g) * u;
-    } else {
-      g = fminf(g, limit);
-      u = fminf(fmaxf(u, -limit), limit);
-      r = g * sigmoid_f(alpha * g) * (u + 1.f);
-    }
-    o[e] = float_to_bf16_bits(r);
+    o[e] = float_to_bf16_bits(glu_value(bf16_bits_to_float(gv[e]),
+                                        bf16_bits_to_float(uv[e]), mode, limit,
+                                        alpha));
   }
-  *reinterpret_cast<ushort8*>(out + i) = o;
+  *reinterpret_cast<ushort8*>(out + t * ldo + c) = o;
 }
 
 }  // namespace arks
@@ -489,20 +488,21 @@ extern "C" void arks_seq_head_norm_gate(void* out, int64_t ldo, const void* o,
       ldo, (const float*)o, (const AT*)gate, ldg, eps, V, out_scale));
 }
 
-extern "C" void arks_seq_glu_act(void* out, const void* gu, int64_t ldg,
-                                 int64_t rows, int F, int mode, float limit,
-                                 float alpha, int act_f32,
+extern "C" void arks_seq_glu_act(void* out, int64_t ldo, const void* gu,
+                                 int64_t ldg, int64_t rows, int F, int mode,
+                                 float limit, float alpha, int act_f32,
                                  hipStream_t stream) {
   const int64_t n = rows * F;
   if (n == 0) return;
-  if (!act_f32 && F % 8 == 0 && ldg % 8 == 0) {
+  if (!act_f32 && F % 8 == 0 && ldg % 8 == 0 && ldo % 8 == 0 &&
+      ((uintptr_t)out & 15) == 0 && ((uintptr_t)gu & 15) == 0) {
     hipLaunchKernelGGL(glu_act_vec8_kernel,
                        dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0,
-                       stream, (bf16*)out, (const bf16*)gu, ldg, rows, F, mode,
-                       limit, alpha);
+                       stream, (bf16*)out, ldo, (const bf16*)gu, ldg, rows, F,
+                       mode, limit, alpha);
     return;
   }
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
       (glu_act_kernel<AT>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
-      stream, (AT*)out, (const AT*)gu, ldg, rows, F, mode, limit, alpha));
+      stream, (AT*)out, ldo, (const AT*)gu, ldg, rows, F, mode, limit, alpha));
 }
