@@ -68,6 +68,29 @@ def rotate(x, pos, base, dims, interleaved):
 
 
 # ------------------------------------------------------------------ mixers
+def attend(q, k, v, scale, size=None, keep=0, cap=0.0, sink=None):
+    """q [n, H, D], k [n, G, D], v [n, G, V] -> [n, H, V]. Row i sees j <= i
+    with i - j < size or j < keep (size None: every j <= i); scores
+    cap * tanh(s / cap) when cap > 0; sink [H]: exp(sink_h) joins the
+    denominator."""
+    n, H, _ = q.shape
+    G = k.shape[1]
+    out = torch.zeros(n, H, v.shape[2], dtype=F64)
+    for i in range(n):
+        seen = [j for j in range(i + 1)
+                if size is None or i - j < size or j < keep]
+        for hh in range(H):
+            g = hh // (H // G)
+            s = (k[seen, g] @ q[i, hh]) * scale
+            if cap > 0:
+                s = cap * torch.tanh(s / cap)
+            mx = s.max() if sink is None else torch.maximum(s.max(), sink[hh])
+            e = torch.exp(s - mx)
+            den = e.sum() + (0.0 if sink is None else torch.exp(sink[hh] - mx))
+            out[i, hh] = (e / den) @ v[seen, g]
+    return out
+
+
 def window_attention(h, w, m):
     """Grouped-query softmax attention: half-split rotary on the first
     rot.dims dims, tanh-capped scores, row i sees j <= i with
@@ -80,17 +103,8 @@ def window_attention(h, w, m):
     v = (h @ w["v"].T).view(n, G, V)
     q = rotate(q, pos, m["rot"]["base"], m["rot"]["dims"], False)
     k = rotate(k, pos, m["rot"]["base"], m["rot"]["dims"], False)
-    cap = float(m["softcap"])
-    size, keep = int(m["mask"]["size"]), int(m["mask"]["keep_first"])
-    out = torch.zeros(n, H, V, dtype=F64)
-    for i in range(n):
-        seen = [j for j in range(i + 1) if i - j < size or j < keep]
-        for hh in range(H):
-            g = hh // (H // G)
-            s = (k[seen, g] @ q[i, hh]) * m["scale"]
-            s = cap * torch.tanh(s / cap)
-            p = torch.softmax(s, 0)
-            out[i, hh] = p @ v[seen, g]
+    out = attend(q, k, v, m["scale"], int(m["mask"]["size"]),
+                 int(m["mask"]["keep_first"]), float(m["softcap"]))
     return out.reshape(n, H * V) @ w["o"].T
 
 
@@ -112,15 +126,9 @@ def latent_attention(h, w, m, eps):
     k_rot = rotate(k_rot, pos, base, R, True)[:, 0]
     k_plain = (c @ w["uk"].T).view(n, H, D)
     v = (c @ w["uv"].T).view(n, H, V)
-    out = torch.zeros(n, H, V, dtype=F64)
-    for i in range(n):
-        for hh in range(H):
-            s = (k_plain[:i + 1, hh] @ q_plain[i, hh]
-                 + k_rot[:i + 1] @ q_rot[i, hh]) * m["scale"]
-            mx = torch.maximum(s.max(), w["sink"][hh])
-            e = torch.exp(s - mx)
-            den = e.sum() + torch.exp(w["sink"][hh] - mx)
-            out[i, hh] = (e / den) @ v[:i + 1, hh]
+    k = torch.cat([k_plain, k_rot[:, None, :].expand(n, H, R)], -1)
+    out = attend(torch.cat([q_plain, q_rot], -1), k, v, m["scale"],
+                 sink=w["sink"])
     return out.reshape(n, H * V) @ w["o"].T
 
 
@@ -137,6 +145,27 @@ def causal_conv(x, taps_w, bias):
     return out
 
 
+def ssm_scan(x, B, C, dt, rate, skip):
+    """x [n, P, V], B and C [n, G, N], dt [n, P], rate and skip [P]:
+    S_h <- exp(-rate_h dt) S_h + dt B x_h^T (N x V), y_h = S_h^T C + skip x."""
+    n, P, V = x.shape
+    G, N = B.shape[1], B.shape[2]
+    y = torch.zeros(n, P, V, dtype=F64)
+    for hh in range(P):
+        g = hh // (P // G)
+        S = torch.zeros(N, V, dtype=F64)
+        for t in range(n):
+            S = torch.exp(-rate[hh] * dt[t, hh]) * S \
+                + dt[t, hh] * torch.outer(B[t, g], x[t, hh])
+            y[t, hh] = S.T @ C[t, g] + skip[hh] * x[t, hh]
+    return y
+
+
+def group_unit_rms(y, parts, eps):
+    n, c = y.shape
+    return unit_rms(y.view(n, parts, c // parts), eps).reshape(n, c)
+
+
 def mamba2(h, w, m, eps):
     n = h.shape[0]
     P, V, N, G = m["heads"], m["vdim"], m["state"], m["groups"]
@@ -149,18 +178,8 @@ def mamba2(h, w, m, eps):
     B = xbc[:, inner:inner + G * N].view(n, G, N)
     C = xbc[:, inner + G * N:].view(n, G, N)
     dt = softplus(p[:, 2 * inner + 2 * G * N:] + w["dt_bias"])  # [n, P]
-    y = torch.zeros(n, P, V, dtype=F64)
-    for hh in range(P):
-        g = hh // (P // G)
-        S = torch.zeros(N, V, dtype=F64)
-        rate = torch.exp(w["A_log"][hh])
-        for t in range(n):
-            S = torch.exp(-rate * dt[t, hh]) * S \
-                + dt[t, hh] * torch.outer(B[t, g], x[t, hh])
-            y[t, hh] = S.T @ C[t, g] + w["D"][hh] * x[t, hh]
-    y = y.reshape(n, inner) * silu(z)
-    parts = m["norm_groups"]
-    y = unit_rms(y.view(n, parts, inner // parts), eps).reshape(n, inner)
+    y = ssm_scan(x, B, C, dt, torch.exp(w["A_log"]), w["D"])
+    y = group_unit_rms(y.reshape(n, inner) * silu(z), m["norm_groups"], eps)
     return (y * w["norm"]) @ w["o"].T
 
 
