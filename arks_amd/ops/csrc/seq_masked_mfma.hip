@@ -1,5 +1,564 @@
-// placeholder until the kernels below are written
+// Masked softmax attention over paged keys on the matrix cores (bf16 rows
+// and pages of 16 tokens, gfx950): the fast path of
+// ops.attention_sink_paged for capped scores, sliding windows that keep the
+// first keys, per-head sinks, and caches whose value is a leading part of
+// the key's row (seq_attention.hip holds the general kernel and the exact
+// definition). Built on the tiling of seq_window_mfma.hip: keys pass
+// through LDS 32 at a time (K rows XOR-swizzled where the row length
+// allows, V as a transposed-read image), both products run on
+// v_mfma_f32_16x16x32_bf16, the softmax is online and fp32.
+//
+// What is new here:
+//   * a tile's 64 score columns are (position, head) pairs: HPT heads of
+//     one key/value head's group side by side for 64 / HPT consecutive
+//     positions. With many query heads on one key/value head (latent
+//     attention has ONE) the keys are staged once for all of them; with one
+//     head per group the tile is 64 positions of that head;
+//   * masks per (column, key): key j for the column at position i iff
+//     j <= i and (i - j < window or j < keep_first); a tile walks the key
+//     tiles that hold kept keys, then those from its oldest row's window on;
+//   * scores may be capped, s <- c tanh(s / c), and the running softmax may
+//     start from a sink (max sink[h], sum 1);
+//   * key and value rows have strides of their own (ldk, ldv);
+//   * no host work list: a workgroup finds its (sequence, first position)
+//     by walking cu_seqlens, or — steps of single rows — from token_seq.
 #include "seq_common.h"
+
+#include <cfloat>
+
+namespace arks {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 mk_bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 mk_bf16x4;
+typedef __attribute__((ext_vector_type(4))) float mk_f32x4;
+
+constexpr int MK_QTILE = 64;
+constexpr int MK_KTILE = 32;
+constexpr int MK_PAGE = 16;
+constexpr int MK_PPAD = 40;
+
+__device__ __forceinline__ float mk_cap(float s, float cap, float inv_cap) {
+  // cap * tanh(s / cap), tanh(z) = 1 - 2 / (e^{2z} + 1)
+  const float z = fminf(fmaxf(s * inv_cap, -15.f), 15.f);
+  return cap * (1.f - 2.f / (__expf(2.f * z) + 1.f));
+}
+
+struct MaskArgs {
+  float scale, softcap, out_scale;
+  int window, keep_first;  // window: INT_MAX / 2 when there is none
+};
+
+template <int D, int V>
+struct MaskedTileLds {
+  static constexpr int K_BYTES = MK_KTILE * D * 2;
+  static constexpr int VT_BYTES = (V / 16) * 8 * 96 * 2;
+  static constexpr int P_BYTES = 4 * 16 * MK_PPAD * 2;
+  static constexpr int BYTES = K_BYTES + VT_BYTES + P_BYTES;
+};
+
+template <int D, int V, bool SINGLE>
+__global__ __launch_bounds__(256) void attn_masked_tile_kernel(
+    bf16* __restrict__ out, int64_t ldo, const bf16* __restrict__ q,
+    const bf16* __restrict__ k_cache, int64_t ldk,
+    const bf16* __restrict__ v_cache, int64_t ldv,
+    const int* __restrict__ block_tables, const int* __restrict__ kv_lens,
+    const int* __restrict__ cu, const int* __restrict__ token_seq,
+    const float* __restrict__ sink_w, int num_seqs, MaskArgs a, int G, int H,
+    int hpt_shift, int max_blocks) {
+  constexpr int STEPS = D / 32;
+  constexpr int CHUNKS = V / 16;
+  constexpr int SWZ = (D % 64 == 0) ? 1 : 0;
+  using Lds = MaskedTileLds<D, V>;
+  extern __shared__ __attribute__((aligned(16))) char mk_smem[];
+  bf16* k_lds = reinterpret_cast<bf16*>(mk_smem);                 // [32][D]
+  bf16* vt_img = reinterpret_cast<bf16*>(mk_smem + Lds::K_BYTES);  // [V/16][8][96]
+  bf16* p_lds = reinterpret_cast<bf16*>(mk_smem + Lds::K_BYTES + Lds::VT_BYTES);
+
+  const int HPT = 1 << hpt_shift;        // heads per tile
+  const int PPT = MK_QTILE >> hpt_shift;  // positions per tile
+  int seq_idx = -1, p0 = 0;
+  if (SINGLE) {
+    seq_idx = token_seq[blockIdx.y];
+    p0 = blockIdx.y - cu[seq_idx];
+  } else {
+    int left = blockIdx.y;
+    for (int s = 0; s < num_seqs; ++s) {
+      const int n = (cu[s + 1] - cu[s] + PPT - 1) / PPT;
+      if (left < n) {
+        seq_idx = s;
+        p0 = left * PPT;
+        break;
+      }
+      left -= n;
+    }
+  }
+  if (seq_idx < 0) return;
+  const int GQ = H / G;
+  const int hblocks = GQ >> hpt_shift;  // head blocks per key/value head
+  const int kvh = blockIdx.x / hblocks;
+  const int h0 = kvh * GQ + (blockIdx.x % hblocks) * HPT;
+  const int q_start = cu[seq_idx];
+  const int q_len = cu[seq_idx + 1] - q_start;
+  const int kv_len = kv_lens[seq_idx];
+  const int kv_off = kv_len - q_len;
+  const int n_pos = SINGLE ? 1 : min(PPT, q_len - p0);
+  const int* __restrict__ bt = block_tables + (int64_t)seq_idx * max_blocks;
+
+  const int tid = threadIdx.x;
+  const int wave = tid / WAVE_SIZE, lane = tid % WAVE_SIZE;
+  const int lq = lane % 16, la = lane / 16;
+
+  // this lane's score column
+  const int col = wave * 16 + lq;
+  const int my_p = col >> hpt_shift;
+  const bool col_valid = my_p < n_pos;
+  const int h = h0 + (col & (HPT - 1));
+  const int my_pos = kv_off + p0 + (col_valid ? my_p : 0);
+  const bool wave_active = wave * 16 < n_pos * HPT;
+  mk_bf16x8 qfrag[STEPS];
+  {
+    const int64_t qbase =
+        ((int64_t)(q_start + p0 + (col_valid ? my_p : 0)) * H + h) * D;
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) {
+      ushort8 u = *reinterpret_cast<const ushort8*>(q + qbase + st * 32 + 8 * la);
+      qfrag[st] = *reinterpret_cast<mk_bf16x8*>(&u);
+    }
+  }
+  const float inv_cap = a.softcap > 0.f ? 1.f / a.softcap : 0.f;
+  float m_run = sink_w ? sink_w[h] : -FLT_MAX;
+  float l_run = sink_w ? 1.f : 0.f;
+  mk_f32x4 oacc[CHUNKS];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) oacc[c] = {0.f, 0.f, 0.f, 0.f};
+
+  const int first_pos = kv_off + p0, last_pos = first_pos + n_pos - 1;
+  const int kmax = last_pos + 1;
+  const int tok_tiles = (kmax + MK_KTILE - 1) / MK_KTILE;
+  const int keep_tiles =
+      (min(a.keep_first, kmax) + MK_KTILE - 1) / MK_KTILE;
+  const int tok_j0 =
+      max(keep_tiles, max(0, first_pos - a.window + 1) / MK_KTILE);
+  const int n_iter = keep_tiles + max(0, tok_tiles - tok_j0);
+
+  for (int it = 0; it < n_iter; ++it) {
+    const int key_base =
+        (it < keep_tiles ? it : tok_j0 + it - keep_tiles) * MK_KTILE;
+    for (int i = tid; i < MK_KTILE * (D / 8); i += 256) {
+      const int key = i / (D / 8);
+      const int col8 = (i % (D / 8)) * 8;
+      const int kg = key_base + key;
+      ushort8 kv{};
+      if (kg < kmax) {
+        const int64_t row =
+            ((int64_t)bt[kg / MK_PAGE] * G + kvh) * MK_PAGE + kg % MK_PAGE;
+        kv = *reinterpret_cast<const ushort8*>(k_cache + row * ldk + col8);
+      }
+      const int swz = (col8 * 2) ^ (SWZ * ((key & 7) << 4));
+      *reinterpret_cast<ushort8*>(
+          reinterpret_cast<char*>(k_lds + key * D) + swz) = kv;
+    }
+    for (int i = tid; i < MK_KTILE * (V / 8); i += 256) {
+      const int key = i / (V / 8);
+      const int col8 = (i % (V / 8)) * 8;
+      const int kg = key_base + key;
+      ushort8 vv{};
+      if (kg < kmax) {
+        const int64_t row =
+            ((int64_t)bt[kg / MK_PAGE] * G + kvh) * MK_PAGE + kg % MK_PAGE;
+        vv = *reinterpret_cast<const ushort8*>(v_cache + row * ldv + col8);
+      }
+      *reinterpret_cast<ushort8*>(
+          &vt_img[((col8 >> 4) * 8 + (key >> 2)) * 96 + (key & 3) * 16 +
+                  (col8 & 15)]) = vv;
+    }
+    __syncthreads();
+
+    if (wave_active) {
+      mk_f32x4 sc[2];
+      sc[0] = {0.f, 0.f, 0.f, 0.f};
+      sc[1] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        const int key = sub * 16 + lq;
+#pragma unroll
+        for (int st = 0; st < STEPS; ++st) {
+          const int col_byte = (st * 32 + 8 * la) * 2;
+          const int swz = col_byte ^ (SWZ * ((key & 7) << 4));
+          ushort8 u = *reinterpret_cast<const ushort8*>(
+              reinterpret_cast<const char*>(k_lds + key * D) + swz);
+          sc[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              *reinterpret_cast<mk_bf16x8*>(&u), qfrag[st], sc[sub], 0, 0, 0);
+        }
+      }
+      float p[8];
+      bool msk[8];
+      float tile_max = -FLT_MAX;
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int kg = key_base + sub * 16 + 4 * la + r;
+          const int i = sub * 4 + r;
+          msk[i] = col_valid && kg <= my_pos &&
+                   (kg > my_pos - a.window || kg < a.keep_first);
+          float s = sc[sub][r] * a.scale;
+          if (a.softcap > 0.f) s = mk_cap(s, a.softcap, inv_cap);
+          p[i] = msk[i] ? s : -FLT_MAX;
+          tile_max = fmaxf(tile_max, p[i]);
+        }
+      }
+      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE_SIZE));
+      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE_SIZE));
+      const float m_new = fmaxf(m_run, tile_max);
+      float alpha = 1.f, psum = 0.f;
+      if (m_new > -FLT_MAX) {
+        alpha = __expf(m_run - m_new);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          p[i] = msk[i] ? __expf(p[i] - m_new) : 0.f;
+          psum += p[i];
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) p[i] = 0.f;
+      }
+      psum += __shfl_xor(psum, 16, WAVE_SIZE);
+      psum += __shfl_xor(psum, 32, WAVE_SIZE);
+      l_run = l_run * alpha + psum;
+      m_run = m_new;
+
+      float row_alpha[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        row_alpha[r] = __shfl(alpha, 4 * la + r, WAVE_SIZE);
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) oacc[c][r] *= row_alpha[r];
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        ushort4v pk;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) pk[r] = float_to_bf16_bits(p[sub * 4 + r]);
+        *reinterpret_cast<ushort4v*>(
+            &p_lds[(wave * 16 + lq) * MK_PPAD + sub * 16 + 4 * la]) = pk;
+      }
+    }
+    __syncthreads();
+
+    if (wave_active) {
+      ushort8 pa = *reinterpret_cast<const ushort8*>(
+          &p_lds[(wave * 16 + lq) * MK_PPAD + 8 * la]);
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c) {
+        mk_bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+            (__attribute__((address_space(3))) mk_bf16x4*)(
+                reinterpret_cast<char*>(&vt_img[(c * 8 + 2 * la) * 96]) + lq * 8));
+        mk_bf16x4 v2 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+            (__attribute__((address_space(3))) mk_bf16x4*)(
+                reinterpret_cast<char*>(&vt_img[(c * 8 + 2 * la + 1) * 96]) +
+                lq * 8));
+        mk_bf16x8 vb;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          vb[e] = v1[e];
+          vb[e + 4] = v2[e];
+        }
+        oacc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            *reinterpret_cast<mk_bf16x8*>(&pa), vb, oacc[c], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+
+  float row_inv[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float lr = __shfl(l_run, 4 * la + r, WAVE_SIZE);
+    row_inv[r] = lr > 0.f ? a.out_scale / lr : 0.f;
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int c2 = wave * 16 + 4 * la + r;  // column of the tile
+    const int pp = c2 >> hpt_shift;
+    if (pp >= n_pos) continue;
+    const int64_t obase = (int64_t)(q_start + p0 + pp) * ldo +
+                          (int64_t)(h0 + (c2 & (HPT - 1))) * V;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+      out[obase + c * 16 + lq] = float_to_bf16_bits(oacc[c][r] * row_inv[r]);
+  }
+}
+
+// Single rows, groups of up to 16 query heads: one workgroup per (row,
+// key/value head) whose four waves each take every fourth visible 32-key
+// tile with no barrier between tiles — K from the pages straight into the
+// MFMA A operand, V through a per-wave transposed-read image, P through a
+// per-wave tile — and merge their (max, sum, output) partials through LDS.
+// The sink, counted once, starts wave 0's running softmax.
+template <int D, int V>
+__global__ __launch_bounds__(256) void attn_masked_dec_kernel(
+    bf16* __restrict__ out, int64_t ldo, const bf16* __restrict__ q,
+    const bf16* __restrict__ k_cache, int64_t ldk,
+    const bf16* __restrict__ v_cache, int64_t ldv,
+    const int* __restrict__ block_tables, const int* __restrict__ kv_lens,
+    const int* __restrict__ cu, const int* __restrict__ token_seq,
+    const float* __restrict__ sink_w, MaskArgs a, int G, int H,
+    int max_blocks) {
+  constexpr int STEPS = D / 32;
+  constexpr int CHUNKS = V / 16;
+  constexpr int E = V / 16;  // value dims per thread in the merge
+  const int t = blockIdx.y, kvh = blockIdx.x;
+  const int GQ = H / G;
+  const int seq = token_seq[t];
+  const int q_start = cu[seq];
+  const int pos = kv_lens[seq] - (cu[seq + 1] - q_start) + (t - q_start);
+  const int* __restrict__ bt = block_tables + (int64_t)seq * max_blocks;
+  const int tid = threadIdx.x;
+  const int wave = tid / WAVE_SIZE, lane = tid % WAVE_SIZE;
+  const int lq = lane % 16, la = lane / 16;
+
+  constexpr int VT_BYTES = (V / 16) * 8 * 96 * 2;
+  constexpr int P_BYTES = 16 * MK_PPAD * 2;
+  constexpr int MERGE_BYTES = 16 * (V + 2) * 4;
+  constexpr int WAVE_BYTES0 =
+      VT_BYTES + P_BYTES > MERGE_BYTES ? VT_BYTES + P_BYTES : MERGE_BYTES;
+  constexpr int WAVE_BYTES = (WAVE_BYTES0 + 15) & ~15;
+  __shared__ __attribute__((aligned(16))) char smem[4][WAVE_BYTES];
+  bf16* vt_lds = reinterpret_cast<bf16*>(smem[wave]);
+  bf16* p_lds = reinterpret_cast<bf16*>(smem[wave] + VT_BYTES);
+  float* merge_lds = reinterpret_cast<float*>(smem[wave]);
+
+  const bool head_valid = lq < GQ;
+  mk_bf16x8 qfrag[STEPS];
+  {
+    const bf16* qp =
+        q + ((int64_t)t * H + kvh * GQ + (head_valid ? lq : 0)) * D;
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) {
+      ushort8 u{};
+      if (head_valid) u = *reinterpret_cast<const ushort8*>(qp + st * 32 + 8 * la);
+      qfrag[st] = *reinterpret_cast<mk_bf16x8*>(&u);
+    }
+  }
+  const float inv_cap = a.softcap > 0.f ? 1.f / a.softcap : 0.f;
+  const bool sunk = sink_w != nullptr && wave == 0 && head_valid;
+  float m_run = sunk ? sink_w[kvh * GQ + lq] : -FLT_MAX;
+  float l_run = sunk ? 1.f : 0.f;
+  mk_f32x4 oacc[CHUNKS];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) oacc[c] = {0.f, 0.f, 0.f, 0.f};
+
+  const int kmax = pos + 1;
+  const int tok_tiles = (kmax + MK_KTILE - 1) / MK_KTILE;
+  const int keep_tiles = (min(a.keep_first, kmax) + MK_KTILE - 1) / MK_KTILE;
+  const int tok_j0 = max(keep_tiles, max(0, pos - a.window + 1) / MK_KTILE);
+  const int n_iter = keep_tiles + max(0, tok_tiles - tok_j0);
+  auto row_of = [&](int kg) -> int64_t {
+    return ((int64_t)bt[kg / MK_PAGE] * G + kvh) * MK_PAGE + kg % MK_PAGE;
+  };
+  constexpr int NV = MK_KTILE * V / 8 / WAVE_SIZE;
+
+  auto load_tile = [&](int it, ushort8 (&kr)[2][STEPS], ushort8 (&vr)[NV]) {
+    const int key_base =
+        (it < keep_tiles ? it : tok_j0 + it - keep_tiles) * MK_KTILE;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int i = lane + WAVE_SIZE * j;
+      const int key = i / (V / 8);
+      const int col8 = (i % (V / 8)) * 8;
+      ushort8 v{};
+      if (key_base + key < kmax)
+        v = *reinterpret_cast<const ushort8*>(
+            v_cache + row_of(key_base + key) * ldv + col8);
+      vr[j] = v;
+    }
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      const int kg = key_base + sub * 16 + lq;
+      const bool have = kg < kmax;
+      const bf16* krow = k_cache + (have ? row_of(kg) : 0) * ldk + 8 * la;
+#pragma unroll
+      for (int st = 0; st < STEPS; ++st) {
+        ushort8 u{};
+        if (have) u = *reinterpret_cast<const ushort8*>(krow + st * 32);
+        kr[sub][st] = u;
+      }
+    }
+  };
+  ushort8 kreg[2][STEPS], vv[NV];
+  if (wave < n_iter) load_tile(wave, kreg, vv);
+
+  for (int it = wave; it < n_iter; it += 4) {
+    const int key_base =
+        (it < keep_tiles ? it : tok_j0 + it - keep_tiles) * MK_KTILE;
+    ushort8 knext[2][STEPS], vnext[NV];
+    if (it + 4 < n_iter) load_tile(it + 4, knext, vnext);
+    mk_f32x4 sc[2];
+    sc[0] = {0.f, 0.f, 0.f, 0.f};
+    sc[1] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int st = 0; st < STEPS; ++st)
+        sc[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            *reinterpret_cast<mk_bf16x8*>(&kreg[sub][st]), qfrag[st], sc[sub],
+            0, 0, 0);
+    float p[8];
+    float tile_max = -FLT_MAX;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int kg = key_base + sub * 16 + 4 * la + r;
+        const int i = sub * 4 + r;
+        const bool vis =
+            kg <= pos && (kg > pos - a.window || kg < a.keep_first);
+        float s = sc[sub][r] * a.scale;
+        if (a.softcap > 0.f) s = mk_cap(s, a.softcap, inv_cap);
+        p[i] = vis ? s : -FLT_MAX;
+        tile_max = fmaxf(tile_max, p[i]);
+      }
+    }
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE_SIZE));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE_SIZE));
+    const float m_new = fmaxf(m_run, tile_max);
+    float alpha = 1.f, psum = 0.f;
+    if (m_new > -FLT_MAX) {
+      alpha = __expf(m_run - m_new);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        p[i] = (p[i] > -FLT_MAX) ? __expf(p[i] - m_new) : 0.f;
+        psum += p[i];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) p[i] = 0.f;
+    }
+    psum += __shfl_xor(psum, 16, WAVE_SIZE);
+    psum += __shfl_xor(psum, 32, WAVE_SIZE);
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    float row_alpha[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) row_alpha[r] = __shfl(alpha, 4 * la + r, WAVE_SIZE);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) oacc[c][r] *= row_alpha[r];
+    // LDS runs in order within a wave: these stores land after the
+    // previous tile's reads
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int i = lane + WAVE_SIZE * j;
+      const int key = i / (V / 8);
+      const int col8 = (i % (V / 8)) * 8;
+      *reinterpret_cast<ushort8*>(
+          &vt_lds[((col8 >> 4) * 8 + (key >> 2)) * 96 + (key & 3) * 16 +
+                  (col8 & 15)]) = vv[j];
+    }
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      ushort4v pk;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) pk[r] = float_to_bf16_bits(p[sub * 4 + r]);
+      *reinterpret_cast<ushort4v*>(&p_lds[lq * MK_PPAD + sub * 16 + 4 * la]) = pk;
+    }
+    // producer -> consumer between lanes of this wave: the LDS counter only
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    ushort8 pa = *reinterpret_cast<const ushort8*>(&p_lds[lq * MK_PPAD + 8 * la]);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      mk_bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+          (__attribute__((address_space(3))) mk_bf16x4*)(
+              reinterpret_cast<char*>(&vt_lds[(c * 8 + 2 * la) * 96]) + lq * 8));
+      mk_bf16x4 v2 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+          (__attribute__((address_space(3))) mk_bf16x4*)(
+              reinterpret_cast<char*>(&vt_lds[(c * 8 + 2 * la + 1) * 96]) + lq * 8));
+      mk_bf16x8 vb;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        vb[e] = v1[e];
+        vb[e + 4] = v2[e];
+      }
+      oacc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+          *reinterpret_cast<mk_bf16x8*>(&pa), vb, oacc[c], 0, 0, 0);
+    }
+    if (it + 4 < n_iter) {
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+        for (int st = 0; st < STEPS; ++st) kreg[sub][st] = knext[sub][st];
+#pragma unroll
+      for (int j = 0; j < NV; ++j) vv[j] = vnext[j];
+    }
+  }
+
+  __syncthreads();  // every wave is done with its tiles before the union flips
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      merge_lds[(4 * la + r) * (V + 2) + c * 16 + lq] = oacc[c][r];
+  if (la == 0) {
+    merge_lds[lq * (V + 2) + V] = m_run;
+    merge_lds[lq * (V + 2) + V + 1] = l_run;
+  }
+  __syncthreads();
+  // 256 threads = 16 heads x 16 slices of the value dims
+  const int g = tid / 16, lane16 = tid % 16;
+  if (g >= GQ) return;
+  float mf = -FLT_MAX, lf = 0.f, af[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) af[e] = 0.f;
+  for (int w = 0; w < 4; ++w) {
+    const float* wl = reinterpret_cast<const float*>(smem[w]);
+    const float mw = wl[g * (V + 2) + V];
+    const float lw = wl[g * (V + 2) + V + 1];
+    const float mn = fmaxf(mf, mw);
+    const float a1 = __expf(mf - mn), a2 = __expf(mw - mn);
+    lf = lf * a1 + lw * a2;
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      af[e] = af[e] * a1 + wl[g * (V + 2) + lane16 * E + e] * a2;
+    mf = mn;
+  }
+  const float inv = lf > 0.f ? a.out_scale / lf : 0.f;
+  bf16* op = out + (int64_t)t * ldo + (int64_t)(kvh * GQ + g) * V + lane16 * E;
+#pragma unroll
+  for (int e = 0; e < E; ++e) op[e] = float_to_bf16_bits(af[e] * inv);
+}
+
+template <int D, int V, bool SINGLE>
+int launch_masked_tile(dim3 grid, hipStream_t stream, bf16* out, int64_t ldo,
+                       const bf16* q, const bf16* k_cache, int64_t ldk,
+                       const bf16* v_cache, int64_t ldv, const int* bt,
+                       const int* kv_lens, const int* cu, const int* token_seq,
+                       const float* sink_w, int num_seqs, MaskArgs a, int G,
+                       int H, int hpt_shift, int max_blocks) {
+  constexpr int BYTES = MaskedTileLds<D, V>::BYTES;
+  static bool raised = false;
+  if (BYTES > 48 * 1024 && !raised) {
+    if (hipFuncSetAttribute(
+            reinterpret_cast<const void*>(&attn_masked_tile_kernel<D, V, SINGLE>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, BYTES) != hipSuccess)
+      return 1;
+    raised = true;
+  }
+  hipLaunchKernelGGL((attn_masked_tile_kernel<D, V, SINGLE>), grid, dim3(256),
+                     BYTES, stream, out, ldo, q, k_cache, ldk, v_cache, ldv, bt,
+                     kv_lens, cu, token_seq, sink_w, num_seqs, a, G, H,
+                     hpt_shift, max_blocks);
+  return 0;
+}
+
+}  // namespace arks
+
+using namespace arks;
+
+// Returns 1 when no kernel is built for these sizes (the caller then runs
+// the general kernel).
 extern "C" int arks_seq_attn_masked_mfma(
     void* out, int64_t ldo, const void* q, const void* k_cache, int64_t ldk,
     const void* v_cache, int64_t ldv, const void* block_tables,
@@ -7,5 +566,60 @@ extern "C" int arks_seq_attn_masked_mfma(
     const void* sink_w, float softcap, int window, int keep_first,
     float out_scale, int T, int H, int G, int D, int V, int bs, int max_blocks,
     int num_seqs, int single_rows, hipStream_t stream) {
+  if (bs != MK_PAGE || H % G || ldk % 8 || ldv % 8 || ldo % 8 ||
+      ((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) ||
+      ((uintptr_t)v_cache & 15) || ((uintptr_t)out & 15))
+    return 1;
+  if (T == 0) return 0;
+  const int GQ = H / G;
+  MaskArgs a;
+  a.scale = scale;
+  a.softcap = softcap;
+  a.out_scale = out_scale;
+  a.window = window > 0 ? window : (1 << 30);
+  a.keep_first = window > 0 ? keep_first : 0;
+  // heads per tile: the largest power of two, at most 64, that divides the
+  // group
+  int hpt_shift = 0;
+  while (hpt_shift < 6 && GQ % (2 << hpt_shift) == 0) ++hpt_shift;
+  const int ppt = MK_QTILE >> hpt_shift;
+  const dim3 grid_tile(G * (GQ >> hpt_shift),
+                       single_rows ? T : (T + ppt - 1) / ppt + num_seqs);
+#define MK_ARGS                                                               \
+  (bf16*)out, ldo, (const bf16*)q, (const bf16*)k_cache, ldk,                 \
+      (const bf16*)v_cache, ldv, (const int*)block_tables,                    \
+      (const int*)seq_lens, (const int*)cu, (const int*)token_seq,            \
+      (const float*)sink_w
+#define MK_TILE(DD, VV)                                                       \
+  if (D == DD && V == VV) {                                                   \
+    if (single_rows)                                                          \
+      return launch_masked_tile<DD, VV, true>(grid_tile, stream, MK_ARGS,     \
+                                              num_seqs, a, G, H, hpt_shift,   \
+                                              max_blocks);                    \
+    return launch_masked_tile<DD, VV, false>(grid_tile, stream, MK_ARGS,      \
+                                             num_seqs, a, G, H, hpt_shift,    \
+                                             max_blocks);                     \
+  }
+#define MK_DEC(DD, VV)                                                        \
+  if (D == DD && V == VV && single_rows && GQ <= 16) {                        \
+    hipLaunchKernelGGL((attn_masked_dec_kernel<DD, VV>), dim3(G, T),          \
+                       dim3(256), 0, stream, MK_ARGS, a, G, H, max_blocks);   \
+    return 0;                                                                 \
+  }
+  MK_DEC(64, 64)
+  MK_DEC(128, 128)
+  MK_DEC(128, 64)
+  MK_DEC(96, 96)
+  MK_DEC(96, 64)
+  MK_TILE(64, 64)
+  MK_TILE(128, 128)
+  MK_TILE(128, 64)
+  MK_TILE(96, 96)
+  MK_TILE(96, 64)
+  MK_TILE(320, 256)
+  MK_TILE(576, 512)
+#undef MK_TILE
+#undef MK_DEC
+#undef MK_ARGS
   return 1;
 }
