@@ -85,17 +85,19 @@ def linear_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return F.linear(x, w).float()
 
 
-def step_chunks(batch: ForwardBatch, device):
+def step_chunks(batch: ForwardBatch, device, chunk: int = 0):
     """Chunk metadata of this step for the chunk-parallel recurrent prefill
     (None for steps whose rows per sequence all fit one chunk, and inside
-    captured decode graphs)."""
+    captured decode graphs). chunk: rows per chunk (default ops.SCAN_CHUNK)."""
+    chunk = chunk or ops.SCAN_CHUNK
     if (device.type != "cuda" or batch.seq_lens_list is None
-            or batch.max_q_len <= ops.SCAN_CHUNK):
+            or batch.max_q_len <= chunk):
         return None
-    if "scan_chunks" not in batch.tile_cache:
-        batch.tile_cache["scan_chunks"] = ops.scan_chunks(
-            batch.seq_lens_list, device)
-    return batch.tile_cache["scan_chunks"]
+    key = ("scan_chunks", chunk)
+    if key not in batch.tile_cache:
+        batch.tile_cache[key] = ops.scan_chunks(
+            batch.seq_lens_list, device, chunk)
+    return batch.tile_cache[key]
 
 
 def _param(*shape, dtype):
@@ -495,7 +497,18 @@ class LatentAttention(SplitMixer):
     q_h' . c + q_h,rot . k_rot and the softmax-weighted sum of latents is
     multiplied by W_uv,h afterwards. The attention kernels therefore see H
     query heads of size kv_rank + rot_dim on ONE key/value head whose value
-    is the first kv_rank columns of its key row."""
+    is the first kv_rank columns of its key row.
+
+    That form costs kv_rank + rot_dim + kv_rank multiply-adds per (row,
+    head, key), against dim + rot_dim + vdim for per-head keys and values,
+    and pays for a step of few rows over a long context. A step with a long
+    portion (EXPAND_ROWS rows or more of one sequence) therefore takes the
+    other form: the latents of every sequence's context are gathered from
+    the pages and up-projected once into per-head keys and values for the
+    step (temporary pages of the usual layout with a block table of their
+    own), and the same attention kernels run on H key/value heads."""
+
+    EXPAND_ROWS = 192
 
     def __init__(self, width: int, heads: int, dim: int, rot_dim: int,
                  vdim: int, kv_rank: int, q_rank: int, scale: float,
@@ -540,6 +553,10 @@ class LatentAttention(SplitMixer):
             self.dq_norm, self.dkv_norm, self.eps, batch.positions,
             self.inv_freq, ckv, batch.slot_mapping)
         q = linear(cq, self.uq).view(T, H, D + R)
+        if (batch.max_q_len >= self.EXPAND_ROWS
+                and batch.kv_lens_list is not None):
+            self._expanded(q, batch, ckv, out, out_scale)
+            return
         # [H, T, D] x [H, D, rank]: the key up-projection applied to q
         q_abs = torch.bmm(q[..., :D].transpose(0, 1),
                           self.uk.view(H, D, rank))
@@ -555,6 +572,42 @@ class LatentAttention(SplitMixer):
         if out_scale != 1.0:
             o = o * out_scale
         out.unflatten(-1, (H, V)).copy_(o.transpose(0, 1))
+
+
+    def _expanded(self, q, batch: ForwardBatch, ckv, out, out_scale) -> None:
+        T = q.shape[0]
+        H, D, R, V, rank = self.H, self.D, self.R, self.V, self.rank
+        bs = ckv.shape[2]
+        nb = [-(-n // bs) for n in batch.kv_lens_list]
+        key = ("latent_pages", bs)
+        if key not in batch.tile_cache:
+            # the context's pages in sequence order, and the block table
+            # of the temporary pages (consecutive), once per step
+            dev = q.device
+            idx = torch.cat([batch.block_tables[s, :n].long()
+                             for s, n in enumerate(nb)])
+            table = torch.zeros((len(nb), max(nb)), dtype=torch.int32)
+            at = 0
+            for s, n in enumerate(nb):
+                table[s, :n] = torch.arange(at, at + n, dtype=torch.int32)
+                at += n
+            batch.tile_cache[key] = (idx, table.to(dev))
+        idx, table = batch.tile_cache[key]
+        NB = idx.shape[0]
+        lat = ckv[idx]  # [NB, 1, bs, rank + R]
+        c = lat[..., :rank].reshape(NB * bs, rank)
+        kt = torch.empty((NB, H, bs, D + R), dtype=q.dtype, device=q.device)
+        kt[..., :D] = linear(c, self.uk).view(NB, bs, H, D).transpose(1, 2)
+        kt[..., D:] = lat[..., rank:]
+        vt = linear(c, self.uv).view(NB, bs, H, V).transpose(1, 2).contiguous()
+        qf = torch.empty((T, H, D + R), dtype=q.dtype, device=q.device)
+        ops.latent_query(q, q[..., :D].transpose(0, 1).contiguous(),
+                         batch.positions, self.inv_freq, qf)
+        ops.attention_sink_paged(
+            qf, kt, vt, table, batch.seq_lens, batch.cu_seqlens,
+            batch.token_seq, self.scale, False, None, True, batch.max_q_len,
+            batch.positions, sink_w=self.sink, out=out.unflatten(-1, (H, V)),
+            out_scale=out_scale)
 
 
 class Mamba2Mixer(SplitMixer):
@@ -619,7 +672,7 @@ class Mamba2Mixer(SplitMixer):
             xbc, p[:, inner + ch:inner + ch + self.P], self.dt_bias, self.rate,
             self.D, cache["ssm"], batch.cu_seqlens, batch.seq_lens,
             batch.state_slots, self.P, self.V, self.N, self.G,
-            batch.max_q_len, step_chunks(batch, p.device))
+            batch.max_q_len, step_chunks(batch, p.device, ops.MAMBA2_CHUNK))
         ops.gate_group_norm(y, p[:, :inner], self.norm, self.norm_groups,
                             self.eps, out, out_scale)
 

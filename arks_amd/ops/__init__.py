@@ -1095,6 +1095,12 @@ def latent_query(q, q_abs, positions, inv_freq, out):
     return ref.latent_query(q, q_abs, positions, inv_freq, out)
 
 
+# rows per chunk of mamba2's chunk-parallel prefill: a chunk's state
+# (heads x state x vdim floats) is written and read four times, so chunks
+# are long; the scan itself is sequential inside a chunk either way
+MAMBA2_CHUNK = 256
+
+
 def mamba2_scan(xbc, dt_raw, dt_bias, rate, Dp, state, cu_seqlens, seq_lens,
                 state_slots, heads, vdim, nstate, groups, max_q_len=0,
                 chunks=None):
@@ -1107,7 +1113,7 @@ def mamba2_scan(xbc, dt_raw, dt_bias, rate, Dp, state, cu_seqlens, seq_lens,
         T = xbc.shape[0]
         out = torch.empty((T, heads * vdim), dtype=torch.float32,
                           device=xbc.device)
-        if chunks is not None and max_q_len > SCAN_CHUNK:
+        if chunks is not None:
             c = chunks
             part = torch.empty((c["n"], heads, nstate, vdim),
                                dtype=torch.float32, device=xbc.device)

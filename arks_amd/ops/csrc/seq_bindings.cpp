@@ -158,7 +158,8 @@ int arks_seq_attn_masked_mfma(void* out, int64_t ldo, const void* q,
                               int window, int keep_first, float out_scale,
                               int T, int H, int G, int D, int V, int bs,
                               int max_blocks, int num_seqs, int single_rows,
-                              hipStream_t stream);
+                              void* ws, int ksplit, hipStream_t stream);
+int arks_seq_attn_masked_ksplit(int T, int H, int G, int max_blocks);
 int arks_seq_moe_route_grouped(void* weights, void* ids, const void* logits,
                                int T, int E, int top, int groups, int keep,
                                hipStream_t stream);
@@ -1123,13 +1124,23 @@ bool attention_masked_mfma(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
   TORCH_CHECK(block_tables.dim() == 2 &&
               block_tables.size(0) == seq_lens.numel());
   const SeqMeta m = check_meta(cu, seq_lens, nullptr, &token_seq, T);
+  // partial sums of a key-split launch (fp32 [T, H, ksplit, V + 2])
+  int ksplit = 1;
+  Tensor ws;
+  if (single_rows) {
+    ksplit = arks_seq_attn_masked_ksplit(T, H, G, (int)block_tables.size(1));
+    if (ksplit > 1)
+      ws = torch::empty({(int64_t)T * H * ksplit * (V + 2)},
+                        q.options().dtype(torch::kFloat32));
+  }
   return arks_seq_attn_masked_mfma(
              out.data_ptr(), ldo, q.data_ptr(), k_cache.data_ptr(), ldk,
              v_cache.data_ptr(), ldv, block_tables.data_ptr(),
              seq_lens.data_ptr(), cu.data_ptr(), token_seq.data_ptr(),
              (float)scale, sw_p, (float)softcap, (int)window, (int)keep_first,
              (float)out_scale, T, H, G, D, V, bs, (int)block_tables.size(1),
-             m.S, single_rows ? 1 : 0, current_stream()) == 0;
+             m.S, single_rows ? 1 : 0, ksplit > 1 ? ws.data_ptr() : nullptr,
+             ksplit, current_stream()) == 0;
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {

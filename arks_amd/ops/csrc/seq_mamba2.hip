@@ -5,10 +5,9 @@
 // (seq_mamba.hip causal_conv_silu), and the gated group norm behind it.
 // Head h reads group g = h / (P / G) of B and C.
 //
-// Scan: one wave per (sequence or chunk, head, 64 value columns); lane v
-// keeps column S[:, v] in registers, so y needs no reduction across lanes.
-// B and C of MB2_ROWS rows at a time are staged in LDS (every lane reads
-// all of them). With `out` null only the end state and the summed step
+// Scan: lane v keeps (a part of) column S[:, v] in registers, so y needs no
+// reduction across lanes. B and C of MB2_ROWS rows at a time are staged in
+// LDS (every lane reads all of them). With `out` null only the end state and the summed step
 // sizes are produced (pass 1 of the chunk-parallel prefill); the combine
 // kernel then turns every chunk's end-from-zero state into its start state
 // and leaves the sequence's final state in its slot.
@@ -16,10 +15,17 @@
 
 namespace arks {
 
-constexpr int MB2_ROWS = 8;
+constexpr int MB2_ROWS = 16;
 
-template <typename AT, int NREG>
-__global__ __launch_bounds__(64) void mamba2_scan_kernel(
+// One workgroup = SPLIT waves per (sequence or chunk, HP heads of one group,
+// 64 value columns): wave w keeps state rows [w * NR, (w + 1) * NR) of
+// column v of each of its HP heads in lane v's registers; the waves'
+// partial outputs of a block of rows meet in LDS. Heads of one group read
+// the same B and C, so HP > 1 divides the LDS reads per multiply-add (it
+// also halves the waves per SIMD, and measured slower: the launcher uses
+// HP = 1). FULL: N == NR * SPLIT, no bound checks on the rows.
+template <typename AT, int NR, int SPLIT, int HP, bool FULL>
+__global__ __launch_bounds__(64 * SPLIT) void mamba2_scan_kernel(
     float* __restrict__ out, const AT* __restrict__ xbc, int64_t ldx,
     const AT* __restrict__ dt_raw, int64_t ldd,
     const float* __restrict__ dt_bias, const float* __restrict__ rate,
@@ -27,65 +33,139 @@ __global__ __launch_bounds__(64) void mamba2_scan_kernel(
     const int* __restrict__ cu, const int* __restrict__ seq_lens,
     const int* __restrict__ slots, float* __restrict__ dsum, int P, int V,
     int N, int G) {
-  __shared__ float bc_s[MB2_ROWS][2 * NREG];
-  __shared__ float dt_s[MB2_ROWS];
-  const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  constexpr int NTOT = NR * SPLIT;
+  constexpr int THREADS = 64 * SPLIT;
+  __shared__ __attribute__((aligned(16))) float bc_s[MB2_ROWS][2 * NTOT];
+  __shared__ float dt_s[MB2_ROWS][HP];
+  __shared__ float x_s[MB2_ROWS][HP][64];
+  __shared__ float y_s[SPLIT > 1 ? SPLIT : 1][MB2_ROWS][HP][64];
+  const int s = blockIdx.x, h0 = blockIdx.y * HP;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int v = blockIdx.z * 64 + lane;
   const bool live = v < V;
   const int first = cu[s], rows = cu[s + 1] - first;
   if (rows == 0) return;
   const int start = seq_lens[s] - rows;
   const int slot = slots[s];
-  const int g = h / (P / G);
-  const float r = rate[h], bias = dt_bias[h], dskip = Dp[h];
-  float st[NREG];
-  float* sp = state + (((int64_t)(slot < 0 ? 0 : slot) * P + h) * N) * V + v;
+  const int g = h0 / (P / G);
+  const int n0 = wave * NR;
+  float r[HP], dskip[HP], dt_total[HP];
+  float st[HP][NR];
   const bool resume = start > 0 && slot >= 0 && live;
+  float* sp =
+      state + (((int64_t)(slot < 0 ? 0 : slot) * P + h0) * N + n0) * V + v;
 #pragma unroll
-  for (int n = 0; n < NREG; ++n)
-    st[n] = (resume && n < N) ? sp[(int64_t)n * V] : 0.f;
+  for (int hp = 0; hp < HP; ++hp) {
+    r[hp] = rate[h0 + hp];
+    dskip[hp] = Dp[h0 + hp];
+    dt_total[hp] = 0.f;
+#pragma unroll
+    for (int n = 0; n < NR; ++n)
+      st[hp][n] = (resume && n0 + n < N)
+                      ? sp[((int64_t)hp * N + n) * V] : 0.f;
+  }
   const int64_t boff = (int64_t)P * V + (int64_t)g * N;
   const int64_t coff = boff + (int64_t)G * N;
-  float dt_total = 0.f;
   for (int r0 = 0; r0 < rows; r0 += MB2_ROWS) {
     const int nr = min(MB2_ROWS, rows - r0);
     __syncthreads();  // the previous rows' readers are done
-    for (int i = lane; i < nr * 2 * N; i += 64) {
-      const int rr = i / (2 * N), c = i % (2 * N);
+    // without outputs only B is needed
+    const int ncol = out ? 2 * N : N;
+    for (int i = threadIdx.x; i < nr * ncol; i += THREADS) {
+      const int rr = i / ncol, c = i % ncol;
       const AT* row = xbc + (int64_t)(first + r0 + rr) * ldx;
-      bc_s[rr][c < N ? c : NREG + c - N] =
+      bc_s[rr][c < N ? c : NTOT + c - N] =
           Act<AT>::ld(row + (c < N ? boff + c : coff + c - N));
     }
-    if (lane < nr)
-      dt_s[lane] = softplus_f(
-          Act<AT>::ld(dt_raw + (int64_t)(first + r0 + lane) * ldd + h) + bias);
+    // this block's x rows too: a load from memory inside the row loop
+    // would expose its latency once per row
+    for (int i = threadIdx.x; i < nr * HP * 64; i += THREADS) {
+      const int rr = i / (HP * 64), hp = (i / 64) % HP, l = i % 64;
+      const int vv = blockIdx.z * 64 + l;
+      x_s[rr][hp][l] =
+          vv < V ? Act<AT>::ld(xbc + (int64_t)(first + r0 + rr) * ldx +
+                               (int64_t)(h0 + hp) * V + vv) : 0.f;
+    }
+    if (threadIdx.x < nr * HP) {
+      const int rr = threadIdx.x / HP, hp = threadIdx.x % HP;
+      dt_s[rr][hp] = softplus_f(
+          Act<AT>::ld(dt_raw + (int64_t)(first + r0 + rr) * ldd + h0 + hp) +
+          dt_bias[h0 + hp]);
+    }
     __syncthreads();
     for (int rr = 0; rr < nr; ++rr) {
       const int t = first + r0 + rr;
-      const float dt = dt_s[rr];
-      const float a = expf(-r * dt);
-      dt_total += dt;
-      const float xv =
-          live ? Act<AT>::ld(xbc + (int64_t)t * ldx + (int64_t)h * V + v) : 0.f;
-      const float dx = dt * xv;
-      float y = 0.f;
+      float a[HP], dx[HP], xv[HP], y[HP];
 #pragma unroll
-      for (int n = 0; n < NREG; ++n) {
-        if (n < N) {
-          st[n] = a * st[n] + bc_s[rr][n] * dx;
-          y += st[n] * bc_s[rr][NREG + n];
+      for (int hp = 0; hp < HP; ++hp) {
+        const float dt = dt_s[rr][hp];
+        a[hp] = expf(-r[hp] * dt);
+        dt_total[hp] += dt;
+        xv[hp] = x_s[rr][hp][lane];
+        dx[hp] = dt * xv[hp];
+        y[hp] = 0.f;
+      }
+      const float* bs = &bc_s[rr][n0];
+      const float* cs = &bc_s[rr][NTOT + n0];
+      if (out) {
+#pragma unroll
+        for (int n = 0; n < NR; ++n) {
+          if (FULL || n0 + n < N) {
+            const float bn = bs[n], cn = cs[n];
+#pragma unroll
+            for (int hp = 0; hp < HP; ++hp) {
+              st[hp][n] = fmaf(a[hp], st[hp][n], bn * dx[hp]);
+              y[hp] = fmaf(st[hp][n], cn, y[hp]);
+            }
+          }
+        }
+#pragma unroll
+        for (int hp = 0; hp < HP; ++hp) {
+          if (SPLIT == 1) {
+            if (live)
+              out[(int64_t)t * P * V + (int64_t)(h0 + hp) * V + v] =
+                  y[hp] + dskip[hp] * xv[hp];
+          } else {
+            y_s[wave][rr][hp][lane] =
+                wave == 0 ? y[hp] + dskip[hp] * xv[hp] : y[hp];
+          }
+        }
+      } else {
+#pragma unroll
+        for (int n = 0; n < NR; ++n) {
+          if (FULL || n0 + n < N) {
+            const float bn = bs[n];
+#pragma unroll
+            for (int hp = 0; hp < HP; ++hp)
+              st[hp][n] = fmaf(a[hp], st[hp][n], bn * dx[hp]);
+          }
         }
       }
-      if (out && live) out[(int64_t)t * P * V + (int64_t)h * V + v] = y + dskip * xv;
+    }
+    if (SPLIT > 1 && out) {
+      __syncthreads();
+      for (int i = wave; i < nr * HP; i += SPLIT) {
+        const int rr = i / HP, hp = i % HP;
+        float y = 0.f;
+#pragma unroll
+        for (int w = 0; w < SPLIT; ++w) y += y_s[w][rr][hp][lane];
+        if (live)
+          out[(int64_t)(first + r0 + rr) * P * V + (int64_t)(h0 + hp) * V + v] = y;
+      }
     }
   }
   if (slot >= 0 && live) {
 #pragma unroll
-    for (int n = 0; n < NREG; ++n)
-      if (n < N) sp[(int64_t)n * V] = st[n];
+    for (int hp = 0; hp < HP; ++hp)
+#pragma unroll
+      for (int n = 0; n < NR; ++n)
+        if (n0 + n < N) sp[((int64_t)hp * N + n) * V] = st[hp][n];
   }
-  if (dsum && slot >= 0 && lane == 0 && blockIdx.z == 0)
-    dsum[(int64_t)slot * P + h] = dt_total;
+  if (dsum && slot >= 0 && threadIdx.x == 0 && blockIdx.z == 0) {
+#pragma unroll
+    for (int hp = 0; hp < HP; ++hp)
+      dsum[(int64_t)slot * P + h0 + hp] = dt_total[hp];
+  }
 }
 
 // part [chunks, P, N, V]: end states from zero in, start states out; the
@@ -172,18 +252,33 @@ extern "C" int arks_seq_mamba2_scan(
     int P, int V, int N, int G, int act_f32, hipStream_t stream) {
   if (N > 256 || N < 1 || P % G) return 1;
   if (S == 0) return 0;
-  const dim3 grid(S, P, (V + 63) / 64);
-#define MB2_LAUNCH(NR)                                                        \
+  // heads per lane: heads of one group share B and C
+  // measured on gfx950 (16384 rows, 128 heads x 64, state 128): one head
+  // per lane with 32 state rows a lane runs both passes in 4.3 ms; two
+  // heads per lane 5.5 ms, 64 rows a lane 5.8 ms (fewer waves per SIMD)
+  const int hp = 1;
+  const dim3 grid(S, P / hp, (V + 63) / 64);
+#define MB2_ARGS                                                              \
+  (float*)out, (const AT*)xbc, ldx, (const AT*)dt_raw, ldd,                   \
+      (const float*)dt_bias, (const float*)rate, (const float*)Dp,            \
+      (float*)state, (const int*)cu, (const int*)seq_lens, (const int*)slots, \
+      (float*)dsum, P, V, N, G
+#define MB2_LAUNCH3(NR, SPLIT, HP, FULL)                                      \
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(                               \
-      (mamba2_scan_kernel<AT, NR>), grid, dim3(64), 0, stream, (float*)out,   \
-      (const AT*)xbc, ldx, (const AT*)dt_raw, ldd, (const float*)dt_bias,     \
-      (const float*)rate, (const float*)Dp, (float*)state, (const int*)cu,    \
-      (const int*)seq_lens, (const int*)slots, (float*)dsum, P, V, N, G))
-  if (N <= 16) MB2_LAUNCH(16);
-  else if (N <= 64) MB2_LAUNCH(64);
-  else if (N <= 128) MB2_LAUNCH(128);
-  else MB2_LAUNCH(256);
+      (mamba2_scan_kernel<AT, NR, SPLIT, HP, FULL>), grid, dim3(64 * SPLIT),  \
+      0, stream, MB2_ARGS))
+#define MB2_LAUNCH(NR, SPLIT)                                                 \
+  do {                                                                        \
+    if (N == NR * SPLIT) MB2_LAUNCH3(NR, SPLIT, 1, true);                     \
+    else MB2_LAUNCH3(NR, SPLIT, 1, false);                                    \
+  } while (0)
+  if (N <= 16) MB2_LAUNCH(16, 1);
+  else if (N <= 64) MB2_LAUNCH(32, 2);
+  else if (N <= 128) MB2_LAUNCH(32, 4);
+  else MB2_LAUNCH(64, 4);
 #undef MB2_LAUNCH
+#undef MB2_LAUNCH3
+#undef MB2_ARGS
   return 0;
 }
 

@@ -64,10 +64,13 @@ __global__ __launch_bounds__(256) void attn_masked_tile_kernel(
     const int* __restrict__ block_tables, const int* __restrict__ kv_lens,
     const int* __restrict__ cu, const int* __restrict__ token_seq,
     const float* __restrict__ sink_w, int num_seqs, MaskArgs a, int G, int H,
-    int hpt_shift, int max_blocks) {
+    int hpt_shift, int max_blocks, float* __restrict__ ws) {
   constexpr int STEPS = D / 32;
   constexpr int CHUNKS = V / 16;
   constexpr int SWZ = (D % 64 == 0) ? 1 : 0;
+  // gridDim.z > 1: workgroup z takes every gridDim.z-th key tile and leaves
+  // (output sums, max, sum) per column in ws for the combine kernel
+  const int ks = gridDim.z, kz = blockIdx.z;
   using Lds = MaskedTileLds<D, V>;
   extern __shared__ __attribute__((aligned(16))) char mk_smem[];
   bf16* k_lds = reinterpret_cast<bf16*>(mk_smem);                 // [32][D]
@@ -126,8 +129,9 @@ __global__ __launch_bounds__(256) void attn_masked_tile_kernel(
     }
   }
   const float inv_cap = a.softcap > 0.f ? 1.f / a.softcap : 0.f;
-  float m_run = sink_w ? sink_w[h] : -FLT_MAX;
-  float l_run = sink_w ? 1.f : 0.f;
+  const bool sunk = sink_w != nullptr && kz == 0;
+  float m_run = sunk ? sink_w[h] : -FLT_MAX;
+  float l_run = sunk ? 1.f : 0.f;
   mk_f32x4 oacc[CHUNKS];
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) oacc[c] = {0.f, 0.f, 0.f, 0.f};
@@ -141,7 +145,7 @@ __global__ __launch_bounds__(256) void attn_masked_tile_kernel(
       max(keep_tiles, max(0, first_pos - a.window + 1) / MK_KTILE);
   const int n_iter = keep_tiles + max(0, tok_tiles - tok_j0);
 
-  for (int it = 0; it < n_iter; ++it) {
+  for (int it = kz; it < n_iter; it += ks) {
     const int key_base =
         (it < keep_tiles ? it : tok_j0 + it - keep_tiles) * MK_KTILE;
     for (int i = tid; i < MK_KTILE * (D / 8); i += 256) {
@@ -272,6 +276,25 @@ __global__ __launch_bounds__(256) void attn_masked_tile_kernel(
     __syncthreads();
   }
 
+  if (ks > 1) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int c2 = wave * 16 + 4 * la + r;
+      const int pp = c2 >> hpt_shift;
+      const float mr = __shfl(m_run, 4 * la + r, WAVE_SIZE);
+      const float lr = __shfl(l_run, 4 * la + r, WAVE_SIZE);
+      if (pp >= n_pos) continue;
+      float* wp = ws + (((int64_t)(q_start + p0 + pp) * H + h0 +
+                         (c2 & (HPT - 1))) * ks + kz) * (V + 2);
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c) wp[c * 16 + lq] = oacc[c][r];
+      if (lq == 0) {
+        wp[V] = mr;
+        wp[V + 1] = lr;
+      }
+    }
+    return;
+  }
   float row_inv[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -291,6 +314,26 @@ __global__ __launch_bounds__(256) void attn_masked_tile_kernel(
   }
 }
 
+// Merge the key-split partials of one (row, head): ws [T, H, ks, V + 2].
+__global__ __launch_bounds__(64) void attn_masked_combine_kernel(
+    bf16* __restrict__ out, int64_t ldo, const float* __restrict__ ws, int H,
+    int V, int ks, float out_scale) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const float* wp = ws + ((int64_t)t * H + h) * ks * (V + 2);
+  float m = -FLT_MAX;
+  for (int z = 0; z < ks; ++z) m = fmaxf(m, wp[z * (V + 2) + V]);
+  float l = 0.f;
+  for (int z = 0; z < ks; ++z)
+    l += wp[z * (V + 2) + V + 1] * __expf(wp[z * (V + 2) + V] - m);
+  const float inv = l > 0.f ? out_scale / l : 0.f;
+  for (int d = threadIdx.x; d < V; d += 64) {
+    float acc = 0.f;
+    for (int z = 0; z < ks; ++z)
+      acc += wp[z * (V + 2) + d] * __expf(wp[z * (V + 2) + V] - m);
+    out[(int64_t)t * ldo + (int64_t)h * V + d] = float_to_bf16_bits(acc * inv);
+  }
+}
+
 // Single rows, groups of up to 16 query heads: one workgroup per (row,
 // key/value head) whose four waves each take every fourth visible 32-key
 // tile with no barrier between tiles — K from the pages straight into the
@@ -298,7 +341,7 @@ __global__ __launch_bounds__(256) void attn_masked_tile_kernel(
 // per-wave tile — and merge their (max, sum, output) partials through LDS.
 // The sink, counted once, starts wave 0's running softmax.
 template <int D, int V>
-__global__ __launch_bounds__(256) void attn_masked_dec_kernel(
+__global__ __launch_bounds__(256, 2) void attn_masked_dec_kernel(
     bf16* __restrict__ out, int64_t ldo, const bf16* __restrict__ q,
     const bf16* __restrict__ k_cache, int64_t ldk,
     const bf16* __restrict__ v_cache, int64_t ldv,
@@ -536,7 +579,7 @@ int launch_masked_tile(dim3 grid, hipStream_t stream, bf16* out, int64_t ldo,
                        const bf16* v_cache, int64_t ldv, const int* bt,
                        const int* kv_lens, const int* cu, const int* token_seq,
                        const float* sink_w, int num_seqs, MaskArgs a, int G,
-                       int H, int hpt_shift, int max_blocks) {
+                       int H, int hpt_shift, int max_blocks, float* ws) {
   constexpr int BYTES = MaskedTileLds<D, V>::BYTES;
   static bool raised = false;
   if (BYTES > 48 * 1024 && !raised) {
@@ -549,13 +592,40 @@ int launch_masked_tile(dim3 grid, hipStream_t stream, bf16* out, int64_t ldo,
   hipLaunchKernelGGL((attn_masked_tile_kernel<D, V, SINGLE>), grid, dim3(256),
                      BYTES, stream, out, ldo, q, k_cache, ldk, v_cache, ldv, bt,
                      kv_lens, cu, token_seq, sink_w, num_seqs, a, G, H,
-                     hpt_shift, max_blocks);
+                     hpt_shift, max_blocks, ws);
+  if (grid.z > 1)
+    hipLaunchKernelGGL(attn_masked_combine_kernel, dim3(grid.y, H), dim3(64),
+                       0, stream, out, ldo, ws, H, V, (int)grid.z,
+                       a.out_scale);
   return 0;
+}
+
+// heads per tile: the largest power of two, at most 64, that divides the
+// group of query heads on one key/value head
+static int masked_hpt_shift(int GQ) {
+  int shift = 0;
+  while (shift < 6 && GQ % (2 << shift) == 0) ++shift;
+  return shift;
 }
 
 }  // namespace arks
 
 using namespace arks;
+
+// Steps of single rows through the tile kernel (groups above 16 heads):
+// into how many workgroups a row's key tiles are split so that the launch
+// fills the chip (1: no split, no workspace).
+extern "C" int arks_seq_attn_masked_ksplit(int T, int H, int G,
+                                           int max_blocks) {
+  const int GQ = H / G;
+  if (GQ <= 16) return 1;
+  const int base = G * (GQ >> masked_hpt_shift(GQ)) * T;
+  const int tiles = (max_blocks * MK_PAGE + MK_KTILE - 1) / MK_KTILE;
+  int ks = (512 + base - 1) / base;
+  if (ks > 16) ks = 16;
+  if (ks > tiles / 2) ks = tiles / 2;
+  return ks < 1 ? 1 : ks;
+}
 
 // Returns 1 when no kernel is built for these sizes (the caller then runs
 // the general kernel).
@@ -565,7 +635,7 @@ extern "C" int arks_seq_attn_masked_mfma(
     const void* seq_lens, const void* cu, const void* token_seq, float scale,
     const void* sink_w, float softcap, int window, int keep_first,
     float out_scale, int T, int H, int G, int D, int V, int bs, int max_blocks,
-    int num_seqs, int single_rows, hipStream_t stream) {
+    int num_seqs, int single_rows, void* ws, int ksplit, hipStream_t stream) {
   if (bs != MK_PAGE || H % G || ldk % 8 || ldv % 8 || ldo % 8 ||
       ((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) ||
       ((uintptr_t)v_cache & 15) || ((uintptr_t)out & 15))
@@ -578,13 +648,11 @@ extern "C" int arks_seq_attn_masked_mfma(
   a.out_scale = out_scale;
   a.window = window > 0 ? window : (1 << 30);
   a.keep_first = window > 0 ? keep_first : 0;
-  // heads per tile: the largest power of two, at most 64, that divides the
-  // group
-  int hpt_shift = 0;
-  while (hpt_shift < 6 && GQ % (2 << hpt_shift) == 0) ++hpt_shift;
+  const int hpt_shift = masked_hpt_shift(GQ);
   const int ppt = MK_QTILE >> hpt_shift;
   const dim3 grid_tile(G * (GQ >> hpt_shift),
-                       single_rows ? T : (T + ppt - 1) / ppt + num_seqs);
+                       single_rows ? T : (T + ppt - 1) / ppt + num_seqs,
+                       single_rows && ws && ksplit > 1 ? ksplit : 1);
 #define MK_ARGS                                                               \
   (bf16*)out, ldo, (const bf16*)q, (const bf16*)k_cache, ldk,                 \
       (const bf16*)v_cache, ldv, (const int*)block_tables,                    \
@@ -595,10 +663,10 @@ extern "C" int arks_seq_attn_masked_mfma(
     if (single_rows)                                                          \
       return launch_masked_tile<DD, VV, true>(grid_tile, stream, MK_ARGS,     \
                                               num_seqs, a, G, H, hpt_shift,   \
-                                              max_blocks);                    \
+                                              max_blocks, (float*)ws);        \
     return launch_masked_tile<DD, VV, false>(grid_tile, stream, MK_ARGS,      \
                                              num_seqs, a, G, H, hpt_shift,    \
-                                             max_blocks);                     \
+                                             max_blocks, nullptr);            \
   }
 #define MK_DEC(DD, VV)                                                        \
   if (D == DD && V == VV && single_rows && GQ <= 16) {                        \
@@ -616,6 +684,8 @@ extern "C" int arks_seq_attn_masked_mfma(
   MK_TILE(128, 64)
   MK_TILE(96, 96)
   MK_TILE(96, 64)
+  MK_TILE(64, 32)
+  MK_TILE(192, 128)
   MK_TILE(320, 256)
   MK_TILE(576, 512)
 #undef MK_TILE

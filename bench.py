@@ -51,14 +51,16 @@ def parse_args():
     # through the pinned double-buffer loader (not the synthetic
     # random-init path the serving bench uses).
     # NOT the headline either: prefill and decode throughput of a layer-list
-    # design (Gagorax) at real layer sizes beside the closest llama-family
+    # design (--design) at real layer sizes beside the closest llama-family
     # model cut to the same width and depth, one JSON line per model and
     # phase. --design-only NAME runs one of the two (profiling).
     p.add_argument("--design-bench", action="store_true")
-    p.add_argument("--design-only", choices=["gagorax", "fusolix", "llama"],
+    p.add_argument("--design-only",
+                   choices=["gagorax", "fusolix", "legalix", "llama"],
                    default=None)
     # which layer-list design --design-bench measures beside llama
-    p.add_argument("--design", choices=["gagorax", "fusolix"], default="gagorax")
+    p.add_argument("--design", choices=["gagorax", "fusolix", "legalix"],
+                   default="gagorax")
     p.add_argument("--cold-start", action="store_true")
     p.add_argument("--ckpt-dir", default="/tmp/arks_ckpt")
     return p.parse_args()
@@ -129,7 +131,7 @@ def run_cold_start(args):
 
 
 def run_design_bench(args):
-    """A layer-list design (--design: Gagorax or Fusolix, 8 blocks at the
+    """A layer-list design (--design: Gagorax, Fusolix or Legalix, 8 blocks at the
     sizes of an 8B model) against llama-3-8b cut to 8 layers: prefill
     tokens/s for one long prompt and for a batch of prompts, decode tokens/s
     for a batch at a fixed context. Random weights, synthetic tokens, one

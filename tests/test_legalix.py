@@ -263,7 +263,7 @@ def test_other_sizes(tmp_path, device, dtype, name):
 @pytest.mark.parametrize("device,dtype", [
     pytest.param("cuda", "float32", id="gpu-f32", marks=pytest.mark.gpu),
     pytest.param("cuda", "bfloat16", id="gpu-bf16", marks=pytest.mark.gpu)])
-def test_matrix_core_sizes(tmp_path, device, dtype):
+def test_matrix_core_sizes(tmp_path, device, dtype, monkeypatch):
     """Head sizes the matrix-core attention kernels are built for, prompts
     across 64-row tile edges and chunk edges of the recurrent prefill, a
     window that ends inside a key tile."""
@@ -276,10 +276,35 @@ def test_matrix_core_sizes(tmp_path, device, dtype):
     w = write_checkpoint(tmp_path / "m", cfg)
     t = toks(200, seed=11)
     want = oracle_logits(cfg, w, t)
+    from arks_amd.models.mixers import LatentAttention
+
+    monkeypatch.setattr(LatentAttention, "EXPAND_ROWS", 100)
     eng = make_engine(tmp_path / "m", device, dtype, max_tokens=512)
     plan = [t[:130], t[130:131], t[131:197], t[197:198], t[198:199], t[199:]]
     got = replay(eng, tmp_path, [[("a", p, False)] for p in plan])["a"]
     assert rel_err(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_latent_attention_per_head_form(tmp_path, device, dtype, monkeypatch):
+    """Steps with a long portion up-project the context's latents into
+    per-head keys and values instead of moving the up-projections to the
+    query: same logits, portions of both kinds in one replay, a second
+    request beside it."""
+    from arks_amd.models.mixers import LatentAttention
+
+    monkeypatch.setattr(LatentAttention, "EXPAND_ROWS", 6)
+    cfg = O.make_config([L(), L(heads=2, dim=12, rot_dim=6, vdim=5, kv_rank=9,
+                               q_rank=8, ff=0)], loop=(0, 2, 2))
+    w = write_checkpoint(tmp_path / "m", cfg)
+    ta, tb = toks(60, seed=2), toks(41, seed=3)
+    eng = make_engine(tmp_path / "m", device, dtype)
+    steps = [[("a", ta[:21], False)], [("a", ta[21:24], False), ("b", tb[:30], False)],
+             [("a", ta[24:43], False), ("b", tb[30:31], False)],
+             [("a", ta[43:], True), ("b", tb[31:], True)]]
+    got = replay(eng, tmp_path, steps)
+    assert rel_err(got["a"], oracle_logits(cfg, w, ta)) < TOL[dtype]
+    assert rel_err(got["b"], oracle_logits(cfg, w, tb)) < TOL[dtype]
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
@@ -532,7 +557,8 @@ def test_mamba2_scan_portions(device, dtype, P, V, N, G):
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
     got, at = [], 0
     for rows in (1, 2, 70, 65):
-        chunks = ops.scan_chunks([rows], dev) if dev.type == "cuda" else None
+        chunks = (ops.scan_chunks([rows], dev, 32)
+                  if dev.type == "cuda" and rows > 32 else None)
         got.append(ops.mamba2_scan(
             xbc[at:at + rows].to(dt_).to(dev), dt_raw[at:at + rows].to(dt_).to(dev),
             bias.float().to(dev), rate.float().to(dev), skip.float().to(dev),
