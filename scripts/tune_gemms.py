@@ -42,6 +42,24 @@ def shapes_for(cfg, tp: int = 1):
     ]
 
 
+def hybrid_shapes(cfg):
+    """(name, in, out, bias) of every distinct bf16 projection of a
+    layer-list model (config.HybridModelConfig), read off the model's own
+    fused parameters."""
+    from arks_amd.models import create_model
+
+    model = create_model(cfg, dtype=torch.bfloat16)
+    seen, out = set(), []
+    for name, p in model.named_parameters():
+        if p.dim() != 2 or p.dtype != torch.bfloat16 or name in ("embed",):
+            continue
+        key = (p.shape[1], p.shape[0])
+        if key not in seen:
+            seen.add(key)
+            out.append((name, p.shape[1], p.shape[0], False))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--model", default="qwen2.5-7b")
@@ -52,6 +70,11 @@ def main():
                     help="also tune the MoE strided-batch bmm shapes "
                          "(NN layout, pre-transposed expert weights)")
     ap.add_argument("--out", default="arks_amd/data/tunableop_gfx950.csv")
+    ap.add_argument("--ms", default=None,
+                    help="comma-separated row counts instead of the default "
+                         "decode and prefill sizes")
+    ap.add_argument("--max-ms-per-shape", type=int, default=0,
+                    help="cap on the tuning time of one shape (ms)")
     args = ap.parse_args()
 
     assert torch.cuda.is_available()
@@ -63,9 +86,13 @@ def main():
     if os.path.exists(args.out):
         tunable.read_file(args.out)  # extend the existing table
 
+    if args.max_ms_per_shape:
+        tunable.set_max_tuning_duration(args.max_ms_per_shape)
     cfg = PRESET_CONFIGS[args.model]
     dev = torch.device("cuda")
-    for name, in_f, out_f, bias in shapes_for(cfg, args.tp):
+    shapes = (hybrid_shapes(cfg) if getattr(cfg, "layers", None) is not None
+              else shapes_for(cfg, args.tp))
+    for name, in_f, out_f, bias in shapes:
         w = torch.randn(out_f, in_f, dtype=torch.bfloat16, device=dev) * 0.01
         b = (
             torch.randn(out_f, dtype=torch.bfloat16, device=dev) * 0.01
@@ -73,6 +100,8 @@ def main():
             else None
         )
         ms = DECODE_MS + (PREFILL_MS if name != "lm_head" else [])
+        if args.ms:
+            ms = [int(x) for x in args.ms.split(",")]
         for m in ms:
             x = torch.randn(m, in_f, dtype=torch.bfloat16, device=dev) * 0.01
             F.linear(x, w, b)  # tuning happens on first call per shape

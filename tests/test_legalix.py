@@ -241,6 +241,11 @@ OTHER_SIZES = {
                                        state=9, vdim=10, conv=2)]),
     "mamba2-group-per-head": dict(layers=[M(heads=4, groups=4, norm_groups=8,
                                             state=3, vdim=4, conv=5)]),
+    "odd-everything": dict(layers=[
+        M(heads=2, vdim=7, state=5, groups=1, norm_groups=2, conv=3, ff=50),
+        A(heads=3, kv_heads=1, dim=10, vdim=6, rot_dims=4, ff=0),
+        L(heads=2, dim=6, rot_dim=2, vdim=3, kv_rank=5, q_rank=7, ff=37)],
+        width=44, vocab=97, loop=(0, 3, 2)),
     "mamba2-no-conv-history": dict(layers=[M(conv=1, state=20, vdim=70,
                                              heads=2, groups=1,
                                              norm_groups=5)]),
@@ -252,7 +257,7 @@ OTHER_SIZES = {
 def test_other_sizes(tmp_path, device, dtype, name):
     cfg = O.make_config(**OTHER_SIZES[name])
     w = write_checkpoint(tmp_path / "m", cfg, seed=3)
-    t = toks(38, seed=9)
+    t = toks(38, vocab=cfg["vocab"], seed=9)
     want = oracle_logits(cfg, w, t)
     eng = make_engine(tmp_path / "m", device, dtype)
     steps = [[("a", p, False)] for p in portions(t, [11, 2, 1, 6])]

@@ -499,7 +499,8 @@ def test_cli_flags_map_to_engine_config():
     assert cfg2.enable_prefix_caching is True
 
 
-@pytest.mark.parametrize("preset", ["tiny-gagorax", "tiny-fusolix"])
+@pytest.mark.parametrize("preset", ["tiny-gagorax", "tiny-fusolix",
+                                    "tiny-legalix"])
 def test_layer_list_preset_serves_completions(preset):
     """A layer-list model (recurrent state slots, no prefix reuse) behind
     the same HTTP front: a completion and a streamed chat, twice, so slots
