@@ -601,8 +601,7 @@ class LatentAttention(SplitMixer):
         kt[..., D:] = lat[..., rank:]
         vt = linear(c, self.uv).view(NB, bs, H, V).transpose(1, 2).contiguous()
         qf = torch.empty((T, H, D + R), dtype=q.dtype, device=q.device)
-        ops.latent_query(q, q[..., :D].transpose(0, 1).contiguous(),
-                         batch.positions, self.inv_freq, qf)
+        ops.latent_query(q, None, batch.positions, self.inv_freq, qf)
         ops.attention_sink_paged(
             qf, kt, vt, table, batch.seq_lens, batch.cu_seqlens,
             batch.token_seq, self.scale, False, None, True, batch.max_q_len,

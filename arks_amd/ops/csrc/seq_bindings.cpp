@@ -997,21 +997,25 @@ void latent_prepare(Tensor cqn, Tensor cq, Tensor ckv, Tensor qw, Tensor kw,
                           current_stream());
 }
 
-void latent_query(Tensor out, Tensor q, Tensor q_abs, Tensor positions,
+void latent_query(Tensor out, Tensor q, OptTensor q_abs, Tensor positions,
                   Tensor freq) {
   const int f32 = act_flag(q, "q");
   check_f32(freq, "inv_freq");
   check_i64(positions, "positions");
-  TORCH_CHECK(q.dim() == 3 && q.is_contiguous() && q_abs.dim() == 3 &&
-              q_abs.is_contiguous() && out.dim() == 3 && out.is_contiguous());
+  TORCH_CHECK(q.dim() == 3 && q.is_contiguous() && out.dim() == 3 &&
+              out.is_contiguous());
   const int T = q.size(0), H = q.size(1), P = freq.numel();
-  const int D = q.size(2) - 2 * P, Rk = q_abs.size(2);
-  TORCH_CHECK(D >= 0 && q_abs.size(0) == H && q_abs.size(1) == T &&
-              out.size(0) == T && out.size(1) == H &&
+  const int D = q.size(2) - 2 * P;
+  const int Rk = q_abs.has_value() ? (int)q_abs->size(2) : D;
+  if (q_abs.has_value())
+    TORCH_CHECK(q_abs->dim() == 3 && q_abs->is_contiguous() &&
+                q_abs->size(0) == H && q_abs->size(1) == T &&
+                q_abs->scalar_type() == q.scalar_type());
+  TORCH_CHECK(D >= 0 && out.size(0) == T && out.size(1) == H &&
               out.size(2) == Rk + 2 * P && positions.numel() == T &&
-              q_abs.scalar_type() == q.scalar_type() &&
               out.scalar_type() == q.scalar_type());
-  arks_seq_latent_query(out.data_ptr(), q.data_ptr(), q_abs.data_ptr(),
+  arks_seq_latent_query(out.data_ptr(), q.data_ptr(),
+                        q_abs.has_value() ? q_abs->data_ptr() : nullptr,
                         positions.data_ptr(), freq.data_ptr(), T, H, D, Rk, P,
                         f32, current_stream());
 }

@@ -48,7 +48,7 @@ struct MaskArgs {
   int window, keep_first;  // window: INT_MAX / 2 when there is none
 };
 
-template <int D, int V>
+template <int D, int V>  // V: the value columns one workgroup holds
 struct MaskedTileLds {
   static constexpr int K_BYTES = MK_KTILE * D * 2;
   static constexpr int VT_BYTES = (V / 16) * 8 * 96 * 2;
@@ -56,8 +56,14 @@ struct MaskedTileLds {
   static constexpr int BYTES = K_BYTES + VT_BYTES + P_BYTES;
 };
 
-template <int D, int V, bool SINGLE>
-__global__ __launch_bounds__(256) void attn_masked_tile_kernel(
+// SHR: the value is the leading part of the key's row (one cache, equal
+// strides), so a tile's rows are loaded once.
+// VS > 1: the value columns are cut into VS parts, one workgroup each (all
+// of them compute the scores): long value rows then need fewer registers
+// and less LDS per workgroup, so several fit a CU and hide each other's
+// load latency.
+template <int D, int VFULL, bool SINGLE, bool SHR, int VS>
+__global__ __launch_bounds__(256, VS > 1 ? 2 : 1) void attn_masked_tile_kernel(
     bf16* __restrict__ out, int64_t ldo, const bf16* __restrict__ q,
     const bf16* __restrict__ k_cache, int64_t ldk,
     const bf16* __restrict__ v_cache, int64_t ldv,
@@ -65,9 +71,11 @@ __global__ __launch_bounds__(256) void attn_masked_tile_kernel(
     const int* __restrict__ cu, const int* __restrict__ token_seq,
     const float* __restrict__ sink_w, int num_seqs, MaskArgs a, int G, int H,
     int hpt_shift, int max_blocks, float* __restrict__ ws) {
+  constexpr int V = VFULL / VS;  // this workgroup's value columns
   constexpr int STEPS = D / 32;
   constexpr int CHUNKS = V / 16;
   constexpr int SWZ = (D % 64 == 0) ? 1 : 0;
+  const int voff = (blockIdx.x % VS) * V;
   // gridDim.z > 1: workgroup z takes every gridDim.z-th key tile and leaves
   // (output sums, max, sum) per column in ws for the combine kernel
   const int ks = gridDim.z, kz = blockIdx.z;
@@ -98,8 +106,8 @@ __global__ __launch_bounds__(256) void attn_masked_tile_kernel(
   if (seq_idx < 0) return;
   const int GQ = H / G;
   const int hblocks = GQ >> hpt_shift;  // head blocks per key/value head
-  const int kvh = blockIdx.x / hblocks;
-  const int h0 = kvh * GQ + (blockIdx.x % hblocks) * HPT;
+  const int kvh = (blockIdx.x / VS) / hblocks;
+  const int h0 = kvh * GQ + ((blockIdx.x / VS) % hblocks) * HPT;
   const int q_start = cu[seq_idx];
   const int q_len = cu[seq_idx + 1] - q_start;
   const int kv_len = kv_lens[seq_idx];
@@ -145,38 +153,94 @@ __global__ __launch_bounds__(256) void attn_masked_tile_kernel(
       max(keep_tiles, max(0, first_pos - a.window + 1) / MK_KTILE);
   const int n_iter = keep_tiles + max(0, tok_tiles - tok_j0);
 
-  for (int it = kz; it < n_iter; it += ks) {
-    const int key_base =
-        (it < keep_tiles ? it : tok_j0 + it - keep_tiles) * MK_KTILE;
-    for (int i = tid; i < MK_KTILE * (D / 8); i += 256) {
+  // A tile's rows travel global -> registers -> LDS. The loads of the next
+  // tile are issued right after this tile's rows reach LDS, so they fly
+  // while the tile is computed: with one or two workgroups on a CU nothing
+  // else would hide their latency. The tile's two pages are looked up once.
+  constexpr int KIT = (MK_KTILE * (D / 8) + 255) / 256;
+  constexpr int VIT = SHR ? 1 : (MK_KTILE * (V / 8) + 255) / 256;
+  ushort8 kld[KIT], vld[VIT];
+  auto tile_base = [&](int it) {
+    return (it < keep_tiles ? it : tok_j0 + it - keep_tiles) * MK_KTILE;
+  };
+  auto load_tile = [&](int it) {
+    const int key_base = tile_base(it);
+    const int pg0 = bt[key_base / MK_PAGE];
+    const int pg1 =
+        key_base + MK_PAGE < kmax ? bt[key_base / MK_PAGE + 1] : 0;
+#pragma unroll
+    for (int j = 0; j < KIT; ++j) {
+      const int i = tid + 256 * j;
       const int key = i / (D / 8);
       const int col8 = (i % (D / 8)) * 8;
       const int kg = key_base + key;
       ushort8 kv{};
-      if (kg < kmax) {
+      if (i < MK_KTILE * (D / 8) && kg < kmax) {
         const int64_t row =
-            ((int64_t)bt[kg / MK_PAGE] * G + kvh) * MK_PAGE + kg % MK_PAGE;
+            ((int64_t)(key < MK_PAGE ? pg0 : pg1) * G + kvh) * MK_PAGE +
+            kg % MK_PAGE;
         kv = *reinterpret_cast<const ushort8*>(k_cache + row * ldk + col8);
       }
-      const int swz = (col8 * 2) ^ (SWZ * ((key & 7) << 4));
-      *reinterpret_cast<ushort8*>(
-          reinterpret_cast<char*>(k_lds + key * D) + swz) = kv;
+      kld[j] = kv;
     }
-    for (int i = tid; i < MK_KTILE * (V / 8); i += 256) {
-      const int key = i / (V / 8);
-      const int col8 = (i % (V / 8)) * 8;
-      const int kg = key_base + key;
-      ushort8 vv{};
-      if (kg < kmax) {
-        const int64_t row =
-            ((int64_t)bt[kg / MK_PAGE] * G + kvh) * MK_PAGE + kg % MK_PAGE;
-        vv = *reinterpret_cast<const ushort8*>(v_cache + row * ldv + col8);
+    if (!SHR) {
+#pragma unroll
+      for (int j = 0; j < VIT; ++j) {
+        const int i = tid + 256 * j;
+        const int key = i / (V / 8);
+        const int col8 = (i % (V / 8)) * 8;
+        const int kg = key_base + key;
+        ushort8 vv{};
+        if (i < MK_KTILE * (V / 8) && kg < kmax) {
+          const int64_t row =
+              ((int64_t)(key < MK_PAGE ? pg0 : pg1) * G + kvh) * MK_PAGE +
+              kg % MK_PAGE;
+          vv = *reinterpret_cast<const ushort8*>(v_cache + row * ldv + voff +
+                                                 col8);
+        }
+        vld[j] = vv;
       }
-      *reinterpret_cast<ushort8*>(
-          &vt_img[((col8 >> 4) * 8 + (key >> 2)) * 96 + (key & 3) * 16 +
-                  (col8 & 15)]) = vv;
     }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int j = 0; j < KIT; ++j) {
+      const int i = tid + 256 * j;
+      const int key = i / (D / 8);
+      const int col8 = (i % (D / 8)) * 8;
+      if (i < MK_KTILE * (D / 8)) {
+        const int swz = (col8 * 2) ^ (SWZ * ((key & 7) << 4));
+        *reinterpret_cast<ushort8*>(
+            reinterpret_cast<char*>(k_lds + key * D) + swz) = kld[j];
+        // the value is the leading part of the key's row: no second load
+        if (SHR && col8 >= voff && col8 < voff + V) {
+          const int vc = col8 - voff;
+          *reinterpret_cast<ushort8*>(
+              &vt_img[((vc >> 4) * 8 + (key >> 2)) * 96 + (key & 3) * 16 +
+                      (vc & 15)]) = kld[j];
+        }
+      }
+    }
+    if (!SHR) {
+#pragma unroll
+      for (int j = 0; j < VIT; ++j) {
+        const int i = tid + 256 * j;
+        const int key = i / (V / 8);
+        const int col8 = (i % (V / 8)) * 8;
+        if (i < MK_KTILE * (V / 8))
+          *reinterpret_cast<ushort8*>(
+              &vt_img[((col8 >> 4) * 8 + (key >> 2)) * 96 + (key & 3) * 16 +
+                      (col8 & 15)]) = vld[j];
+      }
+    }
+  };
+  if (kz < n_iter) load_tile(kz);
+
+  for (int it = kz; it < n_iter; it += ks) {
+    const int key_base = tile_base(it);
+    store_tile();
     __syncthreads();
+    if (it + ks < n_iter) load_tile(it + ks);
 
     if (wave_active) {
       mk_f32x4 sc[2];
@@ -285,12 +349,12 @@ __global__ __launch_bounds__(256) void attn_masked_tile_kernel(
       const float lr = __shfl(l_run, 4 * la + r, WAVE_SIZE);
       if (pp >= n_pos) continue;
       float* wp = ws + (((int64_t)(q_start + p0 + pp) * H + h0 +
-                         (c2 & (HPT - 1))) * ks + kz) * (V + 2);
+                         (c2 & (HPT - 1))) * ks + kz) * (VFULL + 2);
 #pragma unroll
-      for (int c = 0; c < CHUNKS; ++c) wp[c * 16 + lq] = oacc[c][r];
-      if (lq == 0) {
-        wp[V] = mr;
-        wp[V + 1] = lr;
+      for (int c = 0; c < CHUNKS; ++c) wp[voff + c * 16 + lq] = oacc[c][r];
+      if (lq == 0 && voff == 0) {
+        wp[VFULL] = mr;
+        wp[VFULL + 1] = lr;
       }
     }
     return;
@@ -307,7 +371,7 @@ __global__ __launch_bounds__(256) void attn_masked_tile_kernel(
     const int pp = c2 >> hpt_shift;
     if (pp >= n_pos) continue;
     const int64_t obase = (int64_t)(q_start + p0 + pp) * ldo +
-                          (int64_t)(h0 + (c2 & (HPT - 1))) * V;
+                          (int64_t)(h0 + (c2 & (HPT - 1))) * VFULL + voff;
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c)
       out[obase + c * 16 + lq] = float_to_bf16_bits(oacc[c][r] * row_inv[r]);
@@ -573,23 +637,26 @@ __global__ __launch_bounds__(256, 2) void attn_masked_dec_kernel(
   for (int e = 0; e < E; ++e) op[e] = float_to_bf16_bits(af[e] * inv);
 }
 
-template <int D, int V, bool SINGLE>
+template <int D, int V, bool SINGLE, bool SHR, int VS>
 int launch_masked_tile(dim3 grid, hipStream_t stream, bf16* out, int64_t ldo,
                        const bf16* q, const bf16* k_cache, int64_t ldk,
                        const bf16* v_cache, int64_t ldv, const int* bt,
                        const int* kv_lens, const int* cu, const int* token_seq,
                        const float* sink_w, int num_seqs, MaskArgs a, int G,
                        int H, int hpt_shift, int max_blocks, float* ws) {
-  constexpr int BYTES = MaskedTileLds<D, V>::BYTES;
+  constexpr int BYTES = MaskedTileLds<D, V / VS>::BYTES;
+  grid.x *= VS;
   static bool raised = false;
   if (BYTES > 48 * 1024 && !raised) {
     if (hipFuncSetAttribute(
-            reinterpret_cast<const void*>(&attn_masked_tile_kernel<D, V, SINGLE>),
+            reinterpret_cast<const void*>(
+                &attn_masked_tile_kernel<D, V, SINGLE, SHR, VS>),
             hipFuncAttributeMaxDynamicSharedMemorySize, BYTES) != hipSuccess)
       return 1;
     raised = true;
   }
-  hipLaunchKernelGGL((attn_masked_tile_kernel<D, V, SINGLE>), grid, dim3(256),
+  hipLaunchKernelGGL((attn_masked_tile_kernel<D, V, SINGLE, SHR, VS>), grid,
+                     dim3(256),
                      BYTES, stream, out, ldo, q, k_cache, ldk, v_cache, ldv, bt,
                      kv_lens, cu, token_seq, sink_w, num_seqs, a, G, H,
                      hpt_shift, max_blocks, ws);
@@ -648,6 +715,7 @@ extern "C" int arks_seq_attn_masked_mfma(
   a.out_scale = out_scale;
   a.window = window > 0 ? window : (1 << 30);
   a.keep_first = window > 0 ? keep_first : 0;
+  const bool shared_rows = v_cache == k_cache && ldv == ldk;
   const int hpt_shift = masked_hpt_shift(GQ);
   const int ppt = MK_QTILE >> hpt_shift;
   const dim3 grid_tile(G * (GQ >> hpt_shift),
@@ -658,15 +726,15 @@ extern "C" int arks_seq_attn_masked_mfma(
       (const bf16*)v_cache, ldv, (const int*)block_tables,                    \
       (const int*)seq_lens, (const int*)cu, (const int*)token_seq,            \
       (const float*)sink_w
-#define MK_TILE(DD, VV)                                                       \
-  if (D == DD && V == VV) {                                                   \
+#define MK_TILE(DD, VV, SHR, VS)                                              \
+  if (D == DD && V == VV && shared_rows == SHR) {                             \
     if (single_rows)                                                          \
-      return launch_masked_tile<DD, VV, true>(grid_tile, stream, MK_ARGS,     \
-                                              num_seqs, a, G, H, hpt_shift,   \
-                                              max_blocks, (float*)ws);        \
-    return launch_masked_tile<DD, VV, false>(grid_tile, stream, MK_ARGS,      \
-                                             num_seqs, a, G, H, hpt_shift,    \
-                                             max_blocks, nullptr);            \
+      return launch_masked_tile<DD, VV, true, SHR, VS>(                       \
+          grid_tile, stream, MK_ARGS, num_seqs, a, G, H, hpt_shift,           \
+          max_blocks, (float*)ws);                                            \
+    return launch_masked_tile<DD, VV, false, SHR, VS>(                        \
+        grid_tile, stream, MK_ARGS, num_seqs, a, G, H, hpt_shift, max_blocks, \
+        nullptr);                                                             \
   }
 #define MK_DEC(DD, VV)                                                        \
   if (D == DD && V == VV && single_rows && GQ <= 16) {                        \
@@ -679,15 +747,16 @@ extern "C" int arks_seq_attn_masked_mfma(
   MK_DEC(128, 64)
   MK_DEC(96, 96)
   MK_DEC(96, 64)
-  MK_TILE(64, 64)
-  MK_TILE(128, 128)
-  MK_TILE(128, 64)
-  MK_TILE(96, 96)
-  MK_TILE(96, 64)
-  MK_TILE(64, 32)
-  MK_TILE(192, 128)
-  MK_TILE(320, 256)
-  MK_TILE(576, 512)
+  MK_TILE(64, 64, false, 1)
+  MK_TILE(128, 128, false, 1)
+  MK_TILE(128, 64, false, 1)
+  MK_TILE(96, 96, false, 1)
+  MK_TILE(96, 64, false, 1)
+  MK_TILE(64, 32, false, 1)
+  MK_TILE(192, 128, false, 1)
+  MK_TILE(96, 64, true, 1)
+  MK_TILE(320, 256, true, 2)
+  MK_TILE(576, 512, true, 4)
 #undef MK_TILE
 #undef MK_DEC
 #undef MK_ARGS

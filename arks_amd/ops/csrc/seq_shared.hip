@@ -140,7 +140,7 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
 }
 
 // out [T, H, Rk + 2P] = [q_abs[h, t, :] | rotated q[t, h, D:]]; one block
-// per row, waves over heads.
+// per row, waves over heads. q_abs null: the first part is q[t, h, :D].
 template <typename AT>
 __global__ __launch_bounds__(256) void latent_query_kernel(
     AT* __restrict__ out, const AT* __restrict__ q,
@@ -151,7 +151,9 @@ __global__ __launch_bounds__(256) void latent_query_kernel(
   const float pos = (float)positions[t];
   for (int hh = wave; hh < H; hh += 4) {
     AT* dst = out + ((int64_t)t * H + hh) * (Rk + 2 * P);
-    const AT* src = q_abs + ((int64_t)hh * T + t) * Rk;
+    // without q_abs the plain part is q's own (Rk == D)
+    const AT* src = q_abs ? q_abs + ((int64_t)hh * T + t) * Rk
+                          : q + ((int64_t)t * H + hh) * (D + 2 * P);
     for (int i = lane; i < Rk; i += 64) dst[i] = src[i];
     const AT* qr = q + ((int64_t)t * H + hh) * (D + 2 * P) + D;
     for (int i = lane; i < P; i += 64) {

@@ -827,11 +827,12 @@ def latent_prepare(cq, ckv, q_norm_w, kv_norm_w, eps, positions, inv_freq,
 
 def latent_query(q, q_abs, positions, inv_freq, out):
     """out [T, H, Rk + 2P] = [q_abs (given as [H, T, Rk]) | the last 2P
-    dims of q [T, H, D + 2P] turned by the row's position, interleaved]."""
-    rank = q_abs.shape[2]
+    dims of q [T, H, D + 2P] turned by the row's position, interleaved].
+    q_abs None: the first part is q's own first D dims."""
     D = q.shape[2] - 2 * inv_freq.numel()
+    rank = q_abs.shape[2] if q_abs is not None else D
     ang = positions.float()[:, None, None] * inv_freq.float()[None, None, :]
-    out[..., :rank] = q_abs.transpose(0, 1)
+    out[..., :rank] = q_abs.transpose(0, 1) if q_abs is not None else q[..., :D]
     out[..., rank:] = _rotate_pairs(q[..., D:].float(), ang, True).to(out.dtype)
     return out
 
