@@ -63,7 +63,9 @@ struct MaskedTileLds {
 // and less LDS per workgroup, so several fit a CU and hide each other's
 // load latency.
 template <int D, int VFULL, bool SINGLE, bool SHR, int VS>
-__global__ __launch_bounds__(256, VS > 1 ? 2 : 1) void attn_masked_tile_kernel(
+__global__ __launch_bounds__(
+    256, VS > 1 ? 2 : (D + VFULL <= 256 ? 3 : (D + VFULL <= 384 ? 2 : 1)))
+void attn_masked_tile_kernel(
     bf16* __restrict__ out, int64_t ldo, const bf16* __restrict__ q,
     const bf16* __restrict__ k_cache, int64_t ldk,
     const bf16* __restrict__ v_cache, int64_t ldv,

@@ -485,7 +485,8 @@ def test_capped_scores(device, dtype):
 @pytest.mark.parametrize("D,V,H,G,shared", [
     (64, 64, 4, 2, False), (128, 128, 8, 1, False), (128, 64, 2, 2, False),
     (96, 96, 3, 1, False), (96, 64, 5, 1, True), (320, 256, 16, 1, True),
-    (576, 512, 16, 1, True)])
+    (576, 512, 16, 1, True), (576, 512, 128, 1, True), (64, 32, 4, 4, False),
+    (192, 128, 4, 4, False), (96, 64, 2, 1, False)])
 def test_masked_matrix_core_kernels_against_general(dtype, D, V, H, G, shared):
     """Random rows through the matrix-core kernels (prompt tiles, single
     rows) and through the general kernel: window edges inside key tiles,
