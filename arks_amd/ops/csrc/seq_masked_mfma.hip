@@ -464,14 +464,27 @@ __global__ __launch_bounds__(256, 2) void attn_masked_dec_kernel(
   const int keep_tiles = (min(a.keep_first, kmax) + MK_KTILE - 1) / MK_KTILE;
   const int tok_j0 = max(keep_tiles, max(0, pos - a.window + 1) / MK_KTILE);
   const int n_iter = keep_tiles + max(0, tok_tiles - tok_j0);
-  auto row_of = [&](int kg) -> int64_t {
-    return ((int64_t)bt[kg / MK_PAGE] * G + kvh) * MK_PAGE + kg % MK_PAGE;
+  // A tile is two pages. Their ids are looked up two tiles ahead of use
+  // and handed to the loads as values: a lookup inside the load would be a
+  // dependent chain (id, then rows) that one tile of compute cannot hide.
+  auto tile_base = [&](int it) {
+    return (it < keep_tiles ? it : tok_j0 + it - keep_tiles) * MK_KTILE;
+  };
+  auto tile_pages = [&](int it, int& p0, int& p1) {
+    const int key_base = tile_base(it);
+    p0 = (it < n_iter && key_base < kmax) ? bt[key_base / MK_PAGE] : 0;
+    p1 = (it < n_iter && key_base + MK_PAGE < kmax)
+             ? bt[key_base / MK_PAGE + 1] : 0;
   };
   constexpr int NV = MK_KTILE * V / 8 / WAVE_SIZE;
 
-  auto load_tile = [&](int it, ushort8 (&kr)[2][STEPS], ushort8 (&vr)[NV]) {
-    const int key_base =
-        (it < keep_tiles ? it : tok_j0 + it - keep_tiles) * MK_KTILE;
+  auto load_tile = [&](int it, int p0, int p1, ushort8 (&kr)[2][STEPS],
+                       ushort8 (&vr)[NV]) {
+    const int key_base = tile_base(it);
+    auto row_of = [&](int key) -> int64_t {  // key within the tile
+      return ((int64_t)(key < MK_PAGE ? p0 : p1) * G + kvh) * MK_PAGE +
+             key % MK_PAGE;
+    };
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int i = lane + WAVE_SIZE * j;
@@ -479,15 +492,15 @@ __global__ __launch_bounds__(256, 2) void attn_masked_dec_kernel(
       const int col8 = (i % (V / 8)) * 8;
       ushort8 v{};
       if (key_base + key < kmax)
-        v = *reinterpret_cast<const ushort8*>(
-            v_cache + row_of(key_base + key) * ldv + col8);
+        v = *reinterpret_cast<const ushort8*>(v_cache + row_of(key) * ldv +
+                                              col8);
       vr[j] = v;
     }
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
-      const int kg = key_base + sub * 16 + lq;
-      const bool have = kg < kmax;
-      const bf16* krow = k_cache + (have ? row_of(kg) : 0) * ldk + 8 * la;
+      const int key = sub * 16 + lq;
+      const bool have = key_base + key < kmax;
+      const bf16* krow = k_cache + (have ? row_of(key) : 0) * ldk + 8 * la;
 #pragma unroll
       for (int st = 0; st < STEPS; ++st) {
         ushort8 u{};
@@ -497,13 +510,19 @@ __global__ __launch_bounds__(256, 2) void attn_masked_dec_kernel(
     }
   };
   ushort8 kreg[2][STEPS], vv[NV];
-  if (wave < n_iter) load_tile(wave, kreg, vv);
+  int cp0, cp1, np0, np1;
+  tile_pages(wave, cp0, cp1);
+  tile_pages(wave + 4, np0, np1);
+  if (wave < n_iter) load_tile(wave, cp0, cp1, kreg, vv);
 
   for (int it = wave; it < n_iter; it += 4) {
-    const int key_base =
-        (it < keep_tiles ? it : tok_j0 + it - keep_tiles) * MK_KTILE;
+    const int key_base = tile_base(it);
+    int nnp0, nnp1;
+    tile_pages(it + 8, nnp0, nnp1);
     ushort8 knext[2][STEPS], vnext[NV];
-    if (it + 4 < n_iter) load_tile(it + 4, knext, vnext);
+    if (it + 4 < n_iter) load_tile(it + 4, np0, np1, knext, vnext);
+    np0 = nnp0;
+    np1 = nnp1;
     mk_f32x4 sc[2];
     sc[0] = {0.f, 0.f, 0.f, 0.f};
     sc[1] = {0.f, 0.f, 0.f, 0.f};
