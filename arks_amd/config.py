@@ -330,7 +330,7 @@ def _legalix_preset(width, vocab, pattern, heads, kv_heads, dim, window,
         if ch == "a":
             spec = {"type": "attention", "mixer": {
                 "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim,
-                "rot": {"base": 500000.0, "dims": dim}, "scale": dim ** -0.5,
+                "rot": {"base": 1000000.0, "dims": dim}, "scale": dim ** -0.5,
                 "softcap": 50.0,
                 "mask": {"size": window, "keep_first": keep_first}}}
         elif ch == "l":
@@ -347,8 +347,8 @@ def _legalix_preset(width, vocab, pattern, heads, kv_heads, dim, window,
         layers.append(spec)
     return HybridModelConfig(
         architecture="Legalix", vocab_size=vocab, hidden_size=width,
-        layers=layers, rms_norm_eps=1e-6, embed_scale=1.0,
-        residual_mult=0.5, loop=loop)
+        layers=layers, rms_norm_eps=1e-5, embed_scale=1.0,
+        residual_mult=2.0 ** -0.5, loop=loop)
 
 
 # Named synthetic configs for benchmarks / tests (random-init weights; no
