@@ -225,7 +225,7 @@ class HybridModelConfig:
         if not loop:
             return None
         out = {k: int(loop[k]) for k in ("start", "stop", "times")}
-        if not (0 <= out["start"] < out["stop"] <= n_layers and out["times"] >= 1):
+        if not (0 <= out["start"] <= out["stop"] <= n_layers and out["times"] >= 0):
             raise ValueError(f"loop {loop!r} does not fit {n_layers} layers")
         return out
 
@@ -237,7 +237,7 @@ class HybridModelConfig:
             return list(range(n)), []
         a, b, times = self.loop["start"], self.loop["stop"], self.loop["times"]
         order, starts = list(range(a)), []
-        for _ in range(times):
+        for _ in range(times if b > a else 0):
             starts.append(len(order))
             order += list(range(a, b))
         return order + list(range(b, n)), starts

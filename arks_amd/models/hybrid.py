@@ -317,7 +317,7 @@ class HybridForCausalLM(nn.Module):
             self.final_norm_alpha = _param(dtype=torch.float32)
             self._wmap["final.norm.b"] = (self.final_norm_b, 0)
             self._wmap["final.norm.alpha"] = (self.final_norm_alpha, 0)
-            if self.loop_starts:
+            if getattr(cfg, "loop", None):
                 self.loop_in = _param(W, 2 * W, dtype=dtype)
                 self._wmap["loop.in"] = (self.loop_in, 0)
         for i, layer in enumerate(self.layers):

@@ -202,7 +202,7 @@ def layer_runs(cfg):
     a, b, times = loop["start"], loop["stop"], loop["times"]
     order = list(range(a))
     marks = set()
-    for _ in range(times):
+    for _ in range(times if b > a else 0):
         marks.add(len(order))
         order += list(range(a, b))
     order += list(range(b, L))

@@ -225,6 +225,7 @@ OTHER_SIZES = {
     "loop-of-one-pass": dict(layers=[L(), M()], loop=(0, 2, 1)),
     "loop-of-one-layer": dict(layers=[A(), M(), L()], loop=(1, 2, 3)),
     "loop-at-the-end": dict(layers=[M(ff=0), A()], loop=(1, 2, 2)),
+    "loop-of-no-pass": dict(layers=[A(), M(), L()], loop=(1, 2, 0)),
     "one-kv-head": dict(layers=[A(heads=6, kv_heads=1, dim=8, vdim=12)]),
     "all-kv-heads": dict(layers=[A(heads=3, kv_heads=3, dim=12, vdim=12,
                                    rot_dims=12)]),
