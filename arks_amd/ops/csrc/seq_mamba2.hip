@@ -240,6 +240,64 @@ __global__ __launch_bounds__(256) void gate_group_norm_kernel(
   }
 }
 
+// bf16 rows, 4 channels per thread (group size % 4 == 0, aligned rows): the
+// gated values of up to 2048 channels of the group stay in registers.
+__global__ __launch_bounds__(256) void gate_group_norm_vec4_kernel(
+    bf16* __restrict__ out, int64_t ldo, const float* __restrict__ y,
+    const bf16* __restrict__ z, int64_t ldz, const float* __restrict__ w,
+    float eps, int C, int groups, float out_scale) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x, grp = blockIdx.y;
+  const int n = C / groups, c0 = grp * n;
+  constexpr int KEEP = 2;
+  float gv[KEEP][4];
+  float ss = 0.f;
+  auto gated = [&](int i, float (&g)[4]) {
+    const float4v yv =
+        *reinterpret_cast<const float4v*>(y + (int64_t)t * C + c0 + i);
+    const ushort4v zv =
+        *reinterpret_cast<const ushort4v*>(z + (int64_t)t * ldz + c0 + i);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) g[e] = yv[e] * silu_f(bf16_bits_to_float(zv[e]));
+  };
+#pragma unroll
+  for (int u = 0; u < KEEP; ++u) {
+    const int i = (threadIdx.x + 256 * u) * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) gv[u][e] = 0.f;
+    if (i < n) {
+      gated(i, gv[u]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += gv[u][e] * gv[u][e];
+    }
+  }
+  for (int i = (threadIdx.x + 256 * KEEP) * 4; i < n; i += 1024) {
+    float g[4];
+    gated(i, g);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss += g[e] * g[e];
+  }
+  ss = block_reduce_sum<256>(ss, scratch);
+  const float rstd = out_scale / sqrtf(ss / (float)n + eps);
+  auto put = [&](int i, const float (&g)[4]) {
+    const float4v wv = *reinterpret_cast<const float4v*>(w + c0 + i);
+    ushort4v o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = float_to_bf16_bits(g[e] * rstd * wv[e]);
+    *reinterpret_cast<ushort4v*>(out + (int64_t)t * ldo + c0 + i) = o;
+  };
+#pragma unroll
+  for (int u = 0; u < KEEP; ++u) {
+    const int i = (threadIdx.x + 256 * u) * 4;
+    if (i < n) put(i, gv[u]);
+  }
+  for (int i = (threadIdx.x + 256 * KEEP) * 4; i < n; i += 1024) {
+    float g[4];
+    gated(i, g);
+    put(i, g);
+  }
+}
+
 }  // namespace arks
 
 using namespace arks;
@@ -301,6 +359,16 @@ extern "C" void arks_seq_gate_group_norm(void* out, int64_t ldo, const void* y,
                                          int groups, float out_scale,
                                          int act_f32, hipStream_t stream) {
   if (T == 0) return;
+  const int n = C / groups;
+  if (!act_f32 && n % 4 == 0 && ldz % 4 == 0 && ldo % 4 == 0 && C % 4 == 0 &&
+      ((uintptr_t)y & 15) == 0 && ((uintptr_t)w & 15) == 0 &&
+      ((uintptr_t)z & 7) == 0 && ((uintptr_t)out & 7) == 0) {
+    hipLaunchKernelGGL(gate_group_norm_vec4_kernel, dim3(T, groups), dim3(256),
+                       0, stream, (bf16*)out, ldo, (const float*)y,
+                       (const bf16*)z, ldz, (const float*)w, eps, C, groups,
+                       out_scale);
+    return;
+  }
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
       (gate_group_norm_kernel<AT>), dim3(T, groups), dim3(256), 0, stream,
       (AT*)out, ldo, (const float*)y, (const AT*)z, ldz, (const float*)w, eps,

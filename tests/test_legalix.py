@@ -282,9 +282,11 @@ def test_matrix_core_sizes(tmp_path, device, dtype, monkeypatch):
     w = write_checkpoint(tmp_path / "m", cfg)
     t = toks(200, seed=11)
     want = oracle_logits(cfg, w, t)
+    from arks_amd import ops
     from arks_amd.models.mixers import LatentAttention
 
     monkeypatch.setattr(LatentAttention, "EXPAND_ROWS", 100)
+    monkeypatch.setattr(ops, "MAMBA2_CHUNK", 64)  # 130 rows: three chunks
     eng = make_engine(tmp_path / "m", device, dtype, max_tokens=512)
     plan = [t[:130], t[130:131], t[131:197], t[197:198], t[198:199], t[199:]]
     got = replay(eng, tmp_path, [[("a", p, False)] for p in plan])["a"]
