@@ -293,6 +293,50 @@ def test_matrix_core_sizes(tmp_path, device, dtype, monkeypatch):
     assert rel_err(got, want) < TOL[dtype]
 
 
+@pytest.mark.parametrize("device,dtype", [
+    pytest.param("cuda", "float32", id="gpu-f32", marks=pytest.mark.gpu),
+    pytest.param("cuda", "bfloat16", id="gpu-bf16", marks=pytest.mark.gpu)])
+def test_matrix_core_sizes_in_mixed_batches(tmp_path, device, dtype, monkeypatch):
+    """The matrix-core kernels with several sequences in a step: prompt
+    tiles of unequal requests, single rows beside portions, windows and
+    kept keys inside key tiles, both latent forms, a looped layer pair,
+    pages and slots taken again by later requests."""
+    from arks_amd.models.mixers import LatentAttention
+
+    monkeypatch.setattr(LatentAttention, "EXPAND_ROWS", 48)
+    cfg = O.make_config(
+        [M(heads=4, vdim=64, state=16, groups=2, norm_groups=2, conv=4),
+         A(heads=4, kv_heads=2, dim=64, vdim=64, rot_dims=32, size=40,
+           keep_first=3),
+         L(heads=4, dim=32, rot_dim=32, vdim=32, kv_rank=64, q_rank=48)],
+        width=64, loop=(1, 3, 2))
+    w = write_checkpoint(tmp_path / "m", cfg)
+    reqs = {c: toks(n, seed=s) for c, n, s in
+            [("a", 150, 1), ("b", 70, 2), ("c", 101, 3), ("d", 9, 4),
+             ("e", 66, 5)]}
+    want = {c: oracle_logits(cfg, w, t) for c, t in reqs.items()}
+    at = {c: 0 for c in reqs}
+    live, waiting, steps = [], list(reqs), []
+    sizes = [67, 1, 1, 50, 2, 1, 33, 1, 90]
+    k = 0
+    while live or waiting:
+        while waiting and len(live) < 3:
+            live.append(waiting.pop(0))
+        step = []
+        for c in list(live):
+            n = min(sizes[k % len(sizes)], len(reqs[c]) - at[c])
+            k += 1
+            step.append((c, reqs[c][at[c]:at[c] + n], at[c] + n == len(reqs[c])))
+            at[c] += n
+            if at[c] == len(reqs[c]):
+                live.remove(c)
+        steps.append(step)
+    eng = make_engine(tmp_path / "m", device, dtype, max_tokens=352)
+    got = replay(eng, tmp_path, steps)
+    for c in reqs:
+        assert rel_err(got[c], want[c]) < TOL[dtype], c
+
+
 @pytest.mark.parametrize("device,dtype", CASES)
 def test_latent_attention_per_head_form(tmp_path, device, dtype, monkeypatch):
     """Steps with a long portion up-project the context's latents into
