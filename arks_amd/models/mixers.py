@@ -756,8 +756,9 @@ def build_mixer(kind: str, m: dict, width: int, eps: float, dtype,
                 width, m["heads"], m["kv_heads"], m["dim"], m["vdim"],
                 m["scale"], m["rot"]["base"], m["rot"]["dims"], eps, dtype,
                 qk_norm=False, sink=False, rotate_values=False,
-                interleaved=False, softcap=m["softcap"],
-                window=m["mask"]["size"], keep_first=m["mask"]["keep_first"],
+                interleaved=False, softcap=m.get("softcap") or 0.0,
+                window=(m.get("mask") or {}).get("size") or 0,
+                keep_first=(m.get("mask") or {}).get("keep_first") or 0,
                 own_projections=own_projections)
         if kind == "latent_attention":
             return LatentAttention(
