@@ -181,8 +181,14 @@ class HybridModelConfig:
     # what the engine asks of any model config
     sliding_window = None
 
-    ARCHITECTURES = ("Gagorax", "Fusolix", "Legalix")
-    MOE_ARCHITECTURES = ("Fusolix",)
+    ARCHITECTURES = ("Gagorax", "Fusolix", "Legalix", "Rivolix")
+    MOE_ARCHITECTURES = ("Fusolix", "Rivolix")
+    # the logits are taken with the embedding table (no "head" tensor)
+    TIED_HEAD_ARCHITECTURES = ("Rivolix",)
+
+    @property
+    def tied_head(self) -> bool:
+        return self.architecture in self.TIED_HEAD_ARCHITECTURES
 
     @property
     def num_local_experts(self) -> int:
@@ -204,6 +210,15 @@ class HybridModelConfig:
                 raise ValueError(f"unknown feed-forward kind {kind!r}")
             layers.append({"type": entry["type"], "mixer": dict(entry["mixer"]),
                            "mlp": dict(mlp) if mlp is not None else None})
+        for i, entry in enumerate(layers):
+            src = entry["mixer"].get("kv_from")
+            if src is not None and not (
+                    0 <= int(src) < i
+                    and layers[int(src)]["type"] == entry["type"]
+                    and layers[int(src)]["mixer"].get("kv_from") is None):
+                raise ValueError(
+                    f"layer {i}: kv_from {src!r} must name an earlier layer "
+                    "of the same type that keeps keys and values of its own")
         return cls(
             architecture=cfg["architecture"],
             vocab_size=int(cfg["vocab"]),
@@ -257,6 +272,8 @@ class HybridModelConfig:
                         "residual_mult": self.residual_mult})
             if self.loop:
                 out["loop"] = dict(self.loop)
+        if self.architecture == "Rivolix":
+            out.pop("logit_scale")
         return out
 
     @property
@@ -349,6 +366,41 @@ def _legalix_preset(width, vocab, pattern, heads, kv_heads, dim, window,
         architecture="Legalix", vocab_size=vocab, hidden_size=width,
         layers=layers, rms_norm_eps=1e-5, embed_scale=1.0,
         residual_mult=2.0 ** -0.5, loop=loop)
+
+
+def _rivolix_preset(width, vocab, pattern, heads, kv_heads, dim, vdim, taps,
+                    k_heads, k_kv_heads, k_dim, experts, top, expert_ff,
+                    shared_ff) -> HybridModelConfig:
+    """pattern: one letter per layer, d (difference attention with keys and
+    values of its own), s (difference attention on the keys and values of
+    the nearest d before it), k (attention whose values are its keys);
+    every layer has the routed feed-forward with a shared expert."""
+    layers, last_d = [], None
+    for i, ch in enumerate(pattern):
+        if ch in "ds":
+            m = {"heads": heads, "kv_heads": kv_heads, "dim": dim,
+                 "vdim": vdim, "conv": taps, "diff": 0.3,
+                 "q_temp": {"coef": 0.1, "every": 1024},
+                 "scale": dim ** -0.5}
+            if ch == "s":
+                m["kv_from"] = last_d
+            else:
+                last_d = i
+            spec = {"type": "attention", "mixer": m}
+        else:
+            spec = {"type": "attention_2", "mixer": {
+                "heads": k_heads, "kv_heads": k_kv_heads, "dim": k_dim,
+                "vdim": k_dim, "scale": k_dim ** -0.5,
+                "rot": {"base": 500000.0, "dims": k_dim // 2,
+                        "scaling": {"factor": 8.0, "original": 8192,
+                                    "fast": 32.0, "slow": 1.0}}}}
+        spec["mlp"] = {"kind": "moe", "expert": {"ff": expert_ff},
+                       "router": {"experts": experts, "top": top},
+                       "shared": {"ff": shared_ff} if shared_ff else None}
+        layers.append(spec)
+    return HybridModelConfig(
+        architecture="Rivolix", vocab_size=vocab, hidden_size=width,
+        layers=layers, rms_norm_eps=1e-6)
 
 
 # Named synthetic configs for benchmarks / tests (random-init weights; no
@@ -645,6 +697,16 @@ PRESET_CONFIGS: dict[str, ModelConfig] = {
     "tiny-legalix": _legalix_preset(
         128, 512, "mal", 4, 2, 32, 24, 3, 4, 16, 8, 24, 32, 40, 4, 16, 8, 2,
         192, loop={"start": 1, "stop": 3, "times": 2}),
+    # Rivolix at the layer sizes of an ~8B model: difference attention with
+    # 16/4 heads of two 128-wide maps over 128-wide values (every second
+    # such layer on its predecessor's keys and values), 4 taps; key-valued
+    # attention 32/8 heads x 128; 16 experts of ff 3584, 4 per row, beside
+    # a shared expert of ff 3584
+    "rivolix-8b-slice": _rivolix_preset(
+        4096, 32000, "dskddskd", 16, 4, 128, 128, 4, 32, 8, 128, 16, 4, 3584,
+        3584),
+    "tiny-rivolix": _rivolix_preset(
+        128, 512, "dsk", 4, 2, 16, 24, 3, 6, 2, 32, 8, 2, 48, 80),
     "tiny-gpu": ModelConfig(  # GPU-test-sized (head_dim 128 kernels)
         architecture="Qwen2ForCausalLM",
         vocab_size=2048,

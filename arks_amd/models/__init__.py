@@ -30,6 +30,13 @@ _REGISTRY = {
     # tokens, latent attention, mamba2; a looped run of layers
     # (models/hybrid.py SharedNormBlock)
     "Legalix": HybridForCausalLM,
+    # layer-list decoder: two RMS norms of one residual in front of a mixer
+    # and routed experts side by side, each result scaled per channel;
+    # two-map difference attention behind short convolutions (optionally on
+    # an earlier layer's keys and values), attention whose values are its
+    # keys; logits through the embedding table (models/hybrid.py
+    # DualNormBlock)
+    "Rivolix": HybridForCausalLM,
 }
 
 

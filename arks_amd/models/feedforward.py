@@ -20,6 +20,19 @@ constants as constructor parameters:
   captured; above it the (row, expert) pairs are sorted by expert and every
   expert runs plain GEMMs on its own segment (its row block of the stacked
   matrix).
+- InputScaledMoE: `experts` small silu-GLU feed-forwards of which every row
+  uses the `top` with the highest sigmoid (or softmax) score; the score
+  multiplies the expert's INPUT, expert(s h), and the results are summed as
+  they are; a shared expert of its own size runs on every row. Since
+  W (s h) = s (W h), the factor is applied to the gate and up projections
+  of h in the activation kernel, in fp32. One matrix holds every gate|up
+  projection, per expert and then the shared one, one matrix [width,
+  experts * ff + shared_ff] every down projection. Up to DENSE_TOKENS rows
+  the step is three GEMMs with data-independent shapes: all gate|up
+  projections, an activation whose factor is 0 for the experts a row does
+  not use (so their columns are exactly 0), and ONE down GEMM over all
+  columns, which sums the chosen experts and the shared one. Above it the
+  (row, expert) pairs are sorted by expert as in GroupedMoE.
 """
 
 from __future__ import annotations
@@ -138,8 +151,88 @@ class GroupedMoE(nn.Module):
         return ops.moe_mix_rows_seq(y, weights, inv.view(T, k).to(torch.int32))
 
 
-def build_feedforward(mlp: dict, width: int, dtype) -> nn.Module:
+class InputScaledMoE(nn.Module):
+    DENSE_TOKENS = 256  # see models/llama_family.py MoEMLP.DENSE_TOKENS
+
+    def __init__(self, width: int, experts: int, ff: int, top: int, dtype,
+                 shared_ff: int = 0, score: str = "sigmoid",
+                 renorm: bool = False):
+        super().__init__()
+        assert 1 <= top <= experts and score in ("sigmoid", "softmax")
+        self.E, self.ff, self.top, self.sff = experts, ff, top, int(shared_ff)
+        self.width, self.score, self.renorm = width, score, renorm
+        self.router = _param(experts, width, dtype=dtype)
+        self.w_gu = _param(experts * 2 * ff + 2 * self.sff, width, dtype=dtype)
+        self.w_down = _param(width, experts * ff + self.sff, dtype=dtype)
+
+    def weight_map(self) -> dict:
+        m = {"router": (self.router, 0)}
+        W, ff, E, sff = self.width, self.ff, self.E, self.sff
+        for e in range(E):
+            m[f"e{e}.gate"] = (self.w_gu, e * 2 * ff)
+            m[f"e{e}.up"] = (self.w_gu, e * 2 * ff + ff)
+            m[f"e{e}.down"] = (self.w_down, 0, e * ff, (W, ff))
+        if sff:
+            m["shared.gate"] = (self.w_gu, E * 2 * ff)
+            m["shared.up"] = (self.w_gu, E * 2 * ff + sff)
+            m["shared.down"] = (self.w_down, 0, E * ff, (W, sff))
+        return m
+
+    def forward(self, h, batch=None, cache=None) -> torch.Tensor:
+        T = h.shape[0]
+        E, ff, sff, k = self.E, self.ff, self.sff, self.top
+        z = linear_f32(h, self.router)  # fp32 logits
+        if T <= self.DENSE_TOKENS:
+            _, _, scale = ops.moe_route_grouped(
+                z, k, 1, 1, self.score, self.renorm, matrix=True)
+            gu = linear(h, self.w_gu)
+            return linear(ops.moe_glu_scaled(gu, scale, E, ff, sff),
+                          self.w_down)
+        weights, ids = ops.moe_route_grouped(z, k, 1, 1, self.score,
+                                             self.renorm)
+        # (row, expert) pairs sorted by expert: every expert runs two plain
+        # GEMMs on its own contiguous segment (one host read of the sizes)
+        flat = ids.reshape(-1).long()
+        order = torch.argsort(flat, stable=True)
+        tok = torch.div(order, k, rounding_mode="floor")
+        counts = torch.bincount(flat, minlength=E).tolist()
+        xs = h[tok]
+        gu = torch.empty((T * k, 2 * ff), dtype=h.dtype, device=h.device)
+        at = 0
+        for e, n in enumerate(counts):
+            if n:
+                torch.mm(xs[at:at + n],
+                         self.w_gu[e * 2 * ff:(e + 1) * 2 * ff].t(),
+                         out=gu[at:at + n])
+            at += n
+        a = ops.glu_act(gu, "swiglu", row_scale=weights.reshape(-1)[order])
+        y = torch.empty((T * k, self.width), dtype=h.dtype, device=h.device)
+        at = 0
+        for e, n in enumerate(counts):
+            if n:
+                torch.mm(a[at:at + n],
+                         self.w_down[:, e * ff:(e + 1) * ff].t(),
+                         out=y[at:at + n])
+            at += n
+        inv = torch.empty_like(order)
+        inv[order] = torch.arange(T * k, device=h.device)
+        shared = None
+        if sff:
+            sa = ops.glu_act(linear(h, self.w_gu[E * 2 * ff:]), "swiglu")
+            shared = linear(sa, self.w_down[:, E * ff:])
+        return ops.moe_mix_rows_seq(y, torch.ones_like(weights),
+                                    inv.view(T, k).to(torch.int32), shared)
+
+
+def build_feedforward(mlp: dict, width: int, dtype, arch: str = "") -> nn.Module:
     kind = mlp.get("kind", "dense")
+    if arch == "Rivolix":
+        if kind != "moe":
+            raise ValueError(f"unknown feed-forward kind {kind!r}")
+        r = mlp["router"]
+        return InputScaledMoE(width, r["experts"], mlp["expert"]["ff"],
+                              r["top"], dtype,
+                              shared_ff=(mlp.get("shared") or {}).get("ff", 0))
     if kind == "dense":
         return ClampedGLU(width, mlp["ff"], mlp["limit"], dtype)
     if kind == "moe":

@@ -47,6 +47,22 @@ Legalix's is:
   glu_act, each writing its columns of one buffer -> ONE GEMM over
   [W_o | W_down], whose fp32 accumulation is the sum of both sublayers.
 
+Rivolix's is:
+  - TWO norms of the same x per layer, RMS norms whose stored weight is the
+    distance from one, one in front of the mixer and one in front of the
+    feed-forward; each branch's result is multiplied per channel (ls1, ls2)
+    where it joins the residual:
+    x += ls1 * mixer(n1(x)) + ls2 * ff(n2(x)) (DualNormBlock)
+  - mixers "attention" (two-map difference attention behind short
+    convolutions; a layer may read an earlier layer's key/value pages) and
+    "attention_2" (values are the keys; rotary with ramp-scaled
+    frequencies, then unit RMS of q and k); feed-forward InputScaledMoE;
+    the logits are taken with the embedding table
+  Kernel plan per layer: residual_pair_norm (adds the previous layer's two
+  results, scaled, to the fp32 residual and writes both normed rows, one
+  pass) -> mixer and feed-forward, each with GEMMs of its own (their
+  inputs differ).
+
 The per-layer cache is a dict of tensors (paged KV for attention, slot
 state for the recurrent mixers and the token shift), allocated by
 allocate_cache() from each mixer's cache_layout(). A sequence that starts at
@@ -78,7 +94,10 @@ class BlockArrangement:
     # "input": layer norm with bias in front of each sublayer, residual in
     # weighted copies, short input convolution (StreamBlock);
     # "shared": one tanh norm in front of both sublayers, which run side by
-    # side (SharedNormBlock)
+    # side (SharedNormBlock);
+    # "dual": two RMS norms of the same rows, one per sublayer, the
+    # sublayers side by side, a per-channel scale on each result
+    # (DualNormBlock)
     norm_place: str = "output"
 
 
@@ -88,6 +107,8 @@ ARRANGEMENTS = {
                                 norm_place="input"),
     "Legalix": BlockArrangement(token_shift=False, gated_residual=False,
                                 norm_place="shared"),
+    "Rivolix": BlockArrangement(token_shift=False, gated_residual=False,
+                                norm_place="dual"),
 }
 
 
@@ -268,6 +289,42 @@ class SharedNormBlock(nn.Module):
         return linear(buf, self.w_out)
 
 
+class DualNormBlock(nn.Module):
+    """x += ls1 * mixer(n1(x)) + ls2 * ff(n2(x)), n_q(x) = x / rms(x) *
+    (1 + norm_q). The sum and both norms are one kernel of the model's
+    forward (ops.residual_pair_norm); this module holds the weights and the
+    two sublayers. kv_from: the layer run whose key/value pages the mixer
+    reads instead of pages of its own."""
+
+    def __init__(self, width: int, spec: dict, eps: float, dtype, arch: str):
+        super().__init__()
+        f32 = torch.float32
+        self.width = width
+        self.mixer = build_mixer(spec["type"], spec["mixer"], width, eps, dtype,
+                                 arch=arch)
+        self.kv_from = spec["mixer"].get("kv_from")
+        self.ffn = (build_feedforward(spec["mlp"], width, dtype, arch)
+                    if spec.get("mlp") is not None else None)
+        self.norm1 = _param(width, dtype=f32)
+        self.ls1 = _param(width, dtype=f32)
+        if self.ffn is not None:
+            self.norm2 = _param(width, dtype=f32)
+            self.ls2 = _param(width, dtype=f32)
+        else:
+            self.norm2 = self.ls2 = None
+
+    def weight_map(self) -> dict:
+        m = {"mix." + k: v for k, v in self.mixer.weight_map().items()}
+        m["norm1"], m["ls1"] = (self.norm1, 0), (self.ls1, 0)
+        if self.ffn is not None:
+            m.update({"mlp." + k: v for k, v in self.ffn.weight_map().items()})
+            m["norm2"], m["ls2"] = (self.norm2, 0), (self.ls2, 0)
+        return m
+
+    def cache_layout(self, block_size: int, dtype) -> dict:
+        return dict(self.mixer.cache_layout(block_size, dtype))
+
+
 class HybridForCausalLM(nn.Module):
     supports_float32 = True
     has_sequence_state = True  # engine: state slots, no prefix reuse
@@ -292,6 +349,11 @@ class HybridForCausalLM(nn.Module):
                 SharedNormBlock(W, spec, cfg.rms_norm_eps, dtype,
                                 cfg.architecture)
                 for spec in cfg.layers)
+        elif arr.norm_place == "dual":
+            self.layers = nn.ModuleList(
+                DualNormBlock(W, spec, cfg.rms_norm_eps, dtype,
+                              cfg.architecture)
+                for spec in cfg.layers)
         else:
             self.layers = nn.ModuleList(
                 HybridBlock(W, spec, cfg.rms_norm_eps, dtype, arr)
@@ -304,9 +366,13 @@ class HybridForCausalLM(nn.Module):
             self.run_order, loop_starts = list(range(len(self.layers))), []
         self.loop_starts = frozenset(loop_starts)
         self.final_norm = _param(W, dtype=torch.float32)
-        self.head = _param(cfg.vocab_size, W, dtype=dtype)
-        self._wmap = {"embed": (self.embed, 0), "head": (self.head, 0),
+        self._wmap = {"embed": (self.embed, 0),
                       "final.norm": (self.final_norm, 0)}
+        if getattr(cfg, "tied_head", False):
+            self.head = self.embed  # logits through the embedding table
+        else:
+            self.head = _param(cfg.vocab_size, W, dtype=dtype)
+            self._wmap["head"] = (self.head, 0)
         if arr.norm_place == "input":
             self.final_norm_b = _param(W, dtype=torch.float32)
             self._wmap["final.norm.b"] = (self.final_norm_b, 0)
@@ -367,6 +433,8 @@ class HybridForCausalLM(nn.Module):
             return self._forward_streams(batch, caches)
         if self.arr.norm_place == "shared":
             return self._forward_shared(batch, caches)
+        if self.arr.norm_place == "dual":
+            return self._forward_dual(batch, caches)
         x = self.embed[batch.input_ids].float()
         for i, layer in enumerate(self.layers):
             layer(x, batch, caches[i], self.dtype)
@@ -453,6 +521,36 @@ class HybridForCausalLM(nn.Module):
                                    self.final_norm, self.final_norm_b, dtype)
         return linear_f32(n, self.head) * cfg.logit_scale
 
+    def _forward_dual(self, batch: ForwardBatch, caches: list) -> torch.Tensor:
+        """Two-norm arrangement: a layer's two results wait until the kernel
+        that norms the next layer's inputs adds them, scaled per channel, to
+        the residual, so each layer costs one pass over the fp32 rows."""
+        cfg, dtype = self.cfg, self.dtype
+        eps = cfg.rms_norm_eps
+        x = self.embed[batch.input_ids].float()
+        pend = (None, None, None, None)  # y1, ls1, y2, ls2
+        for i, layer in enumerate(self.layers):
+            h1, h2 = ops.residual_pair_norm(x, *pend, layer.norm1, layer.norm2,
+                                            eps, dtype)
+            cache = caches[i]
+            if layer.kv_from is not None:
+                src = caches[layer.kv_from]
+                cache = {**cache, "k": src["k"], "v": src["v"]}
+            y1 = layer.mixer(h1, batch, cache)
+            y2 = layer.ffn(h2, batch, None) if layer.ffn is not None else None
+            pend = (y1, layer.ls1, y2, layer.ls2)
+            if self.residual_tap is not None:
+                ops.residual_pair_norm(x, *pend, None, None, eps, dtype)
+                pend = (None, None, None, None)
+                self.residual_tap(i, x)
+        if batch.logits_indices is not None:
+            x = x[batch.logits_indices]
+            pend = tuple(t[batch.logits_indices] if t is not None and j % 2 == 0
+                         else t for j, t in enumerate(pend))
+        n, _ = ops.residual_pair_norm(x, *pend, self.final_norm, None, eps,
+                                      dtype)
+        return linear_f32(n, self.head) * cfg.logit_scale
+
     # ------------------------------------------------------------ weights
     @staticmethod
     def _span(entry, w):
@@ -523,6 +621,15 @@ class HybridForCausalLM(nn.Module):
 
             if leaf.endswith(".alpha"):
                 w = 0.5 + 0.5 * torch.rand(shape, generator=g, device=dev)
+            elif self.arr.norm_place == "dual" and (
+                    leaf.endswith("norm") or leaf in ("norm1", "norm2")):
+                w = rn(0.1)  # stored as the distance from one
+            elif leaf in ("ls1", "ls2"):
+                w = 0.5 + rn(0.1)
+            elif leaf in ("mix.lq1", "mix.lk1", "mix.lq2", "mix.lk2"):
+                w = rn(0.3)
+            elif leaf in ("mix.q.conv", "mix.k.conv", "mix.v.conv"):
+                w = rn(0.5)
             elif leaf.endswith("norm") or leaf in ("norm1", "norm2"):
                 w = 1.0 + rn(0.1)
             elif leaf == "mix.dt_bias":

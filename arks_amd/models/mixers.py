@@ -30,6 +30,16 @@ constructor parameters so that more than one design can use it:
 - Mamba2Mixer: short causal convolution over [x | B | C], one scalar decay
   per head and token, an [state x vdim] fp32 state per head and sequence,
   silu gate, RMS norm in equal groups of channels.
+- SinkRotaryAttention also takes rotary frequencies scaled over a ramp of
+  wavelengths (rot_scaling), a unit RMS of q and k AFTER the rotation
+  (unit_norm_after) and values that are the keys as projected
+  (value_is_key: no value projection).
+- DiffAttention: two softmax maps per head over the same values, combined
+  as a1 - lambda a2 and brought to unit RMS per head; short causal
+  convolutions behind the q, k and v projections (their last inputs are
+  per-sequence state), a query factor that grows with the logarithm of the
+  position, a sigmoid output gate; optionally on the pages of an earlier
+  layer's keys and values.
 
 WindowPoolAttention, RetentionMixer, LatentAttention and Mamba2Mixer are
 "split" mixers: they name the rows of their
@@ -111,6 +121,35 @@ def rotary_inv_freq(base: float, ndims: int) -> torch.Tensor:
                      -2.0 * i / ndims).float()
 
 
+def ramp_scaled_inv_freq(base: float, ndims: int, scaling: dict | None):
+    """(frequencies, factor on cos and sin). scaling {factor, original, fast,
+    slow}: pair i completes original * f_i / 2 pi turns over the original
+    length; with n(t) = ndims ln(original / (2 pi t)) / (2 ln base) the pair
+    index that completes t turns, pairs below lo = floor(n(fast)) keep f_i,
+    pairs above hi = ceil(n(slow)) get f_i / factor, and those between are
+    blended linearly; cos and sin are multiplied by 0.1 ln(factor) + 1.
+    Everything in float64, rounded once."""
+    import math
+
+    i = torch.arange(ndims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64),
+                  -2.0 * i / ndims)
+    if not scaling:
+        return f.float(), 1.0
+    factor = float(scaling["factor"])
+
+    def pair_of(turns):
+        return (ndims * math.log(float(scaling["original"])
+                                 / (2.0 * math.pi * float(turns)))
+                / (2.0 * math.log(float(base))))
+
+    lo = max(math.floor(pair_of(scaling["fast"])), 0)
+    hi = min(math.ceil(pair_of(scaling["slow"])), ndims - 1)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    f = f / factor * ramp + f * (1.0 - ramp)
+    return f.float(), 0.1 * math.log(factor) + 1.0
+
+
 _DECODE_TILES: dict = {}
 
 
@@ -120,10 +159,13 @@ class SinkRotaryAttention(nn.Module):
                  eps: float, dtype, qk_norm: bool = True, sink: bool = True,
                  rotate_values: bool = True, interleaved: bool = True,
                  softcap: float = 0.0, window: int = 0, keep_first: int = 0,
-                 own_projections: bool = True):
+                 own_projections: bool = True, rot_scaling: dict | None = None,
+                 unit_norm_after: bool = False, value_is_key: bool = False):
         super().__init__()
         assert heads % kv_heads == 0 and rot_dims % 2 == 0 and rot_dims <= dim
         assert not rotate_values or vdim % 2 == 0
+        assert not value_is_key or (vdim == dim and not rotate_values)
+        self.unit_norm_after, self.value_is_key = unit_norm_after, value_is_key
         self.H, self.G, self.D, self.V = heads, kv_heads, dim, vdim
         self.scale, self.eps = float(scale), eps
         self.sink, self.interleaved = sink, interleaved
@@ -135,21 +177,25 @@ class SinkRotaryAttention(nn.Module):
         assert not (self.masked and rotate_values)
         self.out_cols = heads * vdim
         if own_projections:
-            self.qkv = _param(heads * dim + kv_heads * (dim + vdim), width,
-                              dtype=dtype)
+            self.qkv = _param(
+                heads * dim + kv_heads * (dim + (0 if value_is_key else vdim)),
+                width, dtype=dtype)
             self.o = _param(width, heads * vdim, dtype=dtype)
         self.q_norm = _param(dim, dtype=torch.float32) if qk_norm else None
         self.k_norm = _param(dim, dtype=torch.float32) if qk_norm else None
-        self.register_buffer("inv_freq_qk", rotary_inv_freq(rot_base, rot_dims),
-                             persistent=False)
+        freqs, self.rot_mag = ramp_scaled_inv_freq(rot_base, rot_dims,
+                                                   rot_scaling)
+        self.register_buffer("inv_freq_qk", freqs, persistent=False)
         self.register_buffer(
             "inv_freq_v",
             rotary_inv_freq(rot_base, vdim) if rotate_values else None,
             persistent=False)
 
     def in_spans(self) -> list:
-        return [("q", self.H * self.D, False), ("k", self.G * self.D, False),
-                ("v", self.G * self.V, False)]
+        spans = [("q", self.H * self.D, False), ("k", self.G * self.D, False)]
+        if not self.value_is_key:
+            spans.append(("v", self.G * self.V, False))
+        return spans
 
     def extra_weights(self) -> dict:
         if self.q_norm is None:
@@ -158,10 +204,28 @@ class SinkRotaryAttention(nn.Module):
 
     def weight_map(self) -> dict:
         H, G, D, V = self.H, self.G, self.D, self.V
-        m = {"q": (self.qkv, 0), "k": (self.qkv, H * D),
-             "v": (self.qkv, H * D + G * D), "o": (self.o, 0)}
+        m = {"q": (self.qkv, 0), "k": (self.qkv, H * D), "o": (self.o, 0)}
+        if not self.value_is_key:
+            m["v"] = (self.qkv, H * D + G * D)
         m.update(self.extra_weights())
         return m
+
+    def _split(self, p):
+        """q, k, v views of the in-projection's rows; the value is the key
+        as projected where the design has no value projection."""
+        H, G, D, V = self.H, self.G, self.D, self.V
+        q = p[:, :H * D].unflatten(-1, (H, D))
+        k = p[:, H * D:(H + G) * D].unflatten(-1, (G, D))
+        if self.value_is_key:
+            return q, k, k
+        return q, k, p[:, (H + G) * D:(H + G) * D + G * V].unflatten(-1, (G, V))
+
+    def _prepare(self, q, k, v, batch: ForwardBatch, cache: dict):
+        return ops.qk_norm_rope_cache(
+            q, k, v, self.q_norm, self.k_norm, self.eps, batch.positions,
+            self.inv_freq_qk, self.inv_freq_v, cache["k"], cache["v"],
+            batch.slot_mapping, self.interleaved, self.rot_mag,
+            self.unit_norm_after)
 
     def cache_layout(self, block_size: int, dtype) -> dict:
         return {"k": ("paged", (self.G, block_size, self.D), dtype),
@@ -196,13 +260,8 @@ class SinkRotaryAttention(nn.Module):
         """p: rows of the in-projection [q | k | v]; writes the head outputs,
         times out_scale, into out [T, H * V] (rows may be strided)."""
         H, G, D, V = self.H, self.G, self.D, self.V
-        q = p[:, :H * D].unflatten(-1, (H, D))
-        k = p[:, H * D:(H + G) * D].unflatten(-1, (G, D))
-        v = p[:, (H + G) * D:(H + G) * D + G * V].unflatten(-1, (G, V))
-        q = ops.qk_norm_rope_cache(
-            q, k, v, self.q_norm, self.k_norm, self.eps, batch.positions,
-            self.inv_freq_qk, self.inv_freq_v, cache["k"], cache["v"],
-            batch.slot_mapping, self.interleaved)
+        q, k, v = self._split(p)
+        q = self._prepare(q, k, v, batch, cache)
         if self.masked:
             ops.attention_sink_paged(
                 q, cache["k"], cache["v"], batch.block_tables, batch.seq_lens,
@@ -229,13 +288,8 @@ class SinkRotaryAttention(nn.Module):
             out = torch.empty((T, H * V), dtype=xs.dtype, device=xs.device)
             self.core(qkv, batch, cache, out, 1.0)
             return linear(out, self.o)
-        q = qkv[:, :H * D].unflatten(-1, (H, D))
-        k = qkv[:, H * D:(H + G) * D].unflatten(-1, (G, D))
-        v = qkv[:, (H + G) * D:].unflatten(-1, (G, V))
-        q = ops.qk_norm_rope_cache(
-            q, k, v, self.q_norm, self.k_norm, self.eps, batch.positions,
-            self.inv_freq_qk, self.inv_freq_v, cache["k"], cache["v"],
-            batch.slot_mapping, self.interleaved)
+        q, k, v = self._split(qkv)
+        q = self._prepare(q, k, v, batch, cache)
         out = ops.attention_sink_paged(
             q, cache["k"], cache["v"], batch.block_tables, batch.seq_lens,
             batch.cu_seqlens, batch.token_seq, self.scale, self.sink,
@@ -676,6 +730,101 @@ class Mamba2Mixer(SplitMixer):
                             self.eps, out, out_scale)
 
 
+class DiffAttention(SplitMixer):
+    """Softmax attention with two maps per head. In-projection rows
+    [q: H*2*D | k: G*2*D | v: G*V | g: H*V], a head's q and a key/value
+    head's k laid out [map 1 | map 2]. Per row: q, k and v pass a causal
+    depthwise convolution over time (taps per channel, no bias, no
+    activation; the last taps-1 projected rows of a sequence are slot
+    state); q is multiplied by 1 + temp_coef ln(floor((p + 1) / temp_every)
+    + 1) at position p; each map is a causal softmax attention of its own,
+    scores q_m . k_m * scale, over the shared values; with
+    lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff, one number per layer,
+    o = a1 - lambda a2 is divided by its root mean square over the head
+    (no weight), multiplied by 1 - diff and by sigmoid(g).
+
+    The pages hold a token's convolved keys with both maps side by side,
+    [pages, G, bs, 2*D], and its convolved values [pages, G, bs, V]; the
+    attention ops read key m of a row for the query heads of map m
+    (ops.attention_sink_paged(maps=2)). shared_kv: the layer has neither k
+    nor v rows; core() is handed the pages of the layer it borrows from."""
+
+    MAPS = 2
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int,
+                 vdim: int, scale: float, diff: float, conv: int,
+                 temp_coef: float, temp_every: int, eps: float, dtype,
+                 shared_kv: bool = False, own_projections: bool = True):
+        super().__init__()
+        assert heads % kv_heads == 0 and conv >= 1
+        self.H, self.G, self.D, self.V = heads, kv_heads, dim, vdim
+        self.scale, self.diff, self.eps = float(scale), float(diff), eps
+        self.taps, self.shared_kv = int(conv), shared_kv
+        self.temp_coef, self.temp_every = float(temp_coef), int(temp_every)
+        M = self.MAPS
+        self.n_q = heads * M * dim
+        self.n_k = 0 if shared_kv else kv_heads * M * dim
+        self.n_v = 0 if shared_kv else kv_heads * vdim
+        self.ch = self.n_q + self.n_k + self.n_v  # convolved channels
+        self.out_cols = heads * vdim
+        f32 = torch.float32
+        self.conv_w = _param(self.ch, self.taps, dtype=f32)
+        for leaf in ("lq1", "lk1", "lq2", "lk2"):
+            setattr(self, leaf, _param(dim, dtype=f32))
+        self.lam = float(diff)
+        self.register_buffer("conv_w_t", torch.zeros(self.taps, self.ch, dtype=f32),
+                             persistent=False)
+        if own_projections:
+            self._make_projections(width, dtype)
+
+    def in_spans(self) -> list:
+        spans = [("q", self.n_q, False)]
+        if not self.shared_kv:
+            spans += [("k", self.n_k, False), ("v", self.n_v, False)]
+        return spans + [("g", self.H * self.V, False)]
+
+    def extra_weights(self) -> dict:
+        m = {"q.conv": (self.conv_w, 0)}
+        if not self.shared_kv:
+            m["k.conv"] = (self.conv_w, self.n_q)
+            m["v.conv"] = (self.conv_w, self.n_q + self.n_k)
+        for leaf in ("lq1", "lk1", "lq2", "lk2"):
+            m[leaf] = (getattr(self, leaf), 0)
+        return m
+
+    def finish_loading(self) -> None:
+        d = {k: getattr(self, k).data.double() for k in ("lq1", "lk1", "lq2", "lk2")}
+        self.lam = float(torch.exp((d["lq1"] * d["lk1"]).sum())
+                         - torch.exp((d["lq2"] * d["lk2"]).sum())) + self.diff
+        self.conv_w_t.copy_(self.conv_w.data.t())
+
+    def cache_layout(self, block_size: int, dtype) -> dict:
+        out = {}
+        if not self.shared_kv:
+            out["k"] = ("paged", (self.G, block_size, self.MAPS * self.D), dtype)
+            out["v"] = ("paged", (self.G, block_size, self.V), dtype)
+        if self.taps > 1:
+            out["conv"] = ("slot", (self.taps - 1, self.ch), torch.float32)
+        return out
+
+    def core(self, p, batch: ForwardBatch, cache: dict, out, out_scale) -> None:
+        assert out_scale == 1.0
+        T = p.shape[0]
+        H, G, D, V, M = self.H, self.G, self.D, self.V, self.MAPS
+        q = ops.conv_qkv_cache(
+            p, self.n_q, self.n_k, self.n_v, self.conv_w, self.conv_w_t,
+            cache.get("conv"), batch.cu_seqlens, batch.seq_lens,
+            batch.state_slots, batch.token_seq, batch.positions,
+            self.temp_coef, self.temp_every, H, G, M, cache["k"], cache["v"],
+            batch.slot_mapping)
+        a = ops.attention_sink_paged(
+            q.view(T, H * M, D), cache["k"], cache["v"], batch.block_tables,
+            batch.seq_lens, batch.cu_seqlens, batch.token_seq, self.scale,
+            False, None, False, batch.max_q_len, batch.positions, maps=M)
+        ops.diff_head_norm_gate(a, p[:, self.ch:self.ch + H * V], self.lam,
+                                self.eps, 1.0 - self.diff, H, G, out)
+
+
 class ParallelMixer(nn.Module):
     """left_scale * left(h) + right_scale * right(h) for two split mixers:
     one GEMM projects h for both, each core() writes its head outputs,
@@ -770,6 +919,28 @@ def build_mixer(kind: str, m: dict, width: int, eps: float, dtype,
                 width, m["heads"], m["vdim"], m["state"], m["groups"],
                 m["norm_groups"], m["conv"], eps, dtype,
                 own_projections=own_projections)
+        raise ValueError(f"unknown mixer type {kind!r}")
+    if arch == "Rivolix":
+        if kind == "attention":
+            temp = m.get("q_temp") or {}
+            return DiffAttention(
+                width, m["heads"], m["kv_heads"], m["dim"], m["vdim"],
+                m["scale"], m["diff"], m["conv"], temp.get("coef", 0.0),
+                temp.get("every", 0), eps, dtype,
+                shared_kv=m.get("kv_from") is not None,
+                own_projections=own_projections)
+        if kind == "attention_2":
+            if m["vdim"] != m["dim"]:
+                raise ValueError("attention_2: the values are the keys, "
+                                 "so vdim must equal dim")
+            rot = m.get("rot") or {"base": 10000.0, "dims": 0}
+            return SinkRotaryAttention(
+                width, m["heads"], m["kv_heads"], m["dim"], m["vdim"],
+                m["scale"], rot["base"], rot["dims"], eps, dtype,
+                qk_norm=False, sink=False, rotate_values=False,
+                interleaved=False, own_projections=own_projections,
+                rot_scaling=rot.get("scaling"), unit_norm_after=True,
+                value_is_key=True)
         raise ValueError(f"unknown mixer type {kind!r}")
     if kind == "attention":
         return SinkRotaryAttention(

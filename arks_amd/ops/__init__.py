@@ -638,17 +638,22 @@ def rms_norm_f32(x, weight, eps, out_dtype):
 
 def qk_norm_rope_cache(q, k, v, q_norm_w, k_norm_w, eps, positions,
                        inv_freq_qk, inv_freq_v, k_cache, v_cache,
-                       slot_mapping, interleaved=True):
+                       slot_mapping, interleaved=True, rot_mag=1.0,
+                       unit_norm_after=False):
+    """rot_mag: factor on cos and sin; unit_norm_after: q and k are divided
+    by their root mean square over the head after the rotation (no weight)."""
     if q.is_cuda:
         T, H, D = q.shape
         qo = torch.empty((T, H, D), dtype=q.dtype, device=q.device)
         _native_seq().qk_norm_rope_cache(
             qo, q, k, v, q_norm_w, k_norm_w, eps, positions, inv_freq_qk,
-            inv_freq_v, k_cache, v_cache, slot_mapping, interleaved)
+            inv_freq_v, k_cache, v_cache, slot_mapping, interleaved,
+            float(rot_mag), bool(unit_norm_after))
         return qo
     return ref.qk_norm_rope_cache(q, k, v, q_norm_w, k_norm_w, eps, positions,
                                   inv_freq_qk, inv_freq_v, k_cache, v_cache,
-                                  slot_mapping, interleaved)
+                                  slot_mapping, interleaved, rot_mag,
+                                  unit_norm_after)
 
 
 # head sizes the MFMA kernels are built for (q/k size == value size)
@@ -671,7 +676,7 @@ def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
                          inv_freq_v=None, interleaved=True, max_q_len=0,
                          positions=None, tiles=None, sink_w=None,
                          softcap=0.0, window=0, keep_first=0, out=None,
-                         out_scale=1.0):
+                         out_scale=1.0, maps=1):
     """Causal attention of packed rows over paged keys with an optional
     sink (score 0, or sink_w per head), tanh-capped scores, a sliding
     window that keeps the first keep_first keys, and position-turned values
@@ -680,9 +685,11 @@ def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
     each row's output back); capped, windowed or per-head-sink attention
     runs the masked matrix-core kernels where they are built; anything else
     — float32 rows, other sizes — runs the general kernel. out: a [T, H, V]
-    view (rows may be strided) to write, times out_scale."""
+    view (rows may be strided) to write, times out_scale. maps M > 1: a key
+    row holds M keys side by side that share the row's value, and query
+    head group g * M + m reads key m of key/value head g."""
     masked = (sink_w is not None or softcap > 0 or window > 0
-              or out is not None
+              or out is not None or maps > 1
               or k_cache.untyped_storage().data_ptr()
               == v_cache.untyped_storage().data_ptr())
     if q.is_cuda and masked:
@@ -695,11 +702,11 @@ def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
                 and S.attention_masked_mfma(
                     out, q, k_cache, v_cache, block_tables, seq_lens,
                     cu_seqlens, token_seq, scale, sink_w, softcap, window,
-                    keep_first, out_scale, max_q_len == 1)):
+                    keep_first, out_scale, max_q_len == 1, maps)):
             S.attention_sink_paged(
                 out, q, k_cache, v_cache, block_tables, seq_lens, cu_seqlens,
                 token_seq, scale, sink, None, interleaved, max_q_len, sink_w,
-                softcap, window, keep_first, out_scale)
+                softcap, window, keep_first, out_scale, maps)
         return out
     if q.is_cuda:
         T, H, D = q.shape
@@ -729,12 +736,12 @@ def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
         _native_seq().attention_sink_paged(
             out, q, k_cache, v_cache, block_tables, seq_lens, cu_seqlens,
             token_seq, scale, sink, inv_freq_v, interleaved, max_q_len, None,
-            0.0, 0, 0, 1.0)
+            0.0, 0, 0, 1.0, 1)
         return out
     res = ref.attention_sink_paged(q, k_cache, v_cache, block_tables,
                                    seq_lens, cu_seqlens, scale, sink,
                                    inv_freq_v, interleaved, sink_w, softcap,
-                                   window, keep_first)
+                                   window, keep_first, maps)
     if out is None:
         return res
     out.copy_((res.float() * out_scale).to(out.dtype))
@@ -1005,34 +1012,45 @@ def head_norm_gate(o, gate, eps, heads, out, out_scale=1.0):
 _GLU_MODES = {"swiglu": 0, "clamped": 1, "gelu_tanh": 2}
 
 
-def glu_act(gu, kind, limit=0.0, alpha=1.0, out=None):
+def glu_act(gu, kind, limit=0.0, alpha=1.0, out=None, row_scale=None):
     """[gate | up] rows -> activated rows (ref.glu_act); out: a [T, F]
-    view (rows may be strided) to write instead of a new tensor."""
+    view (rows may be strided) to write instead of a new tensor; row_scale
+    [T] fp32: a factor on each row's gate and up."""
     if gu.is_cuda:
         F_ = gu.shape[-1] // 2
         if out is None:
             out = torch.empty((gu.shape[0], F_), dtype=gu.dtype,
                               device=gu.device)
         _native_seq().glu_act(out, gu, _GLU_MODES[kind], float(limit),
-                              float(alpha))
+                              float(alpha), row_scale)
         return out
-    res = ref.glu_act(gu, kind, limit, alpha)
+    res = ref.glu_act(gu, kind, limit, alpha, row_scale)
     if out is None:
         return res
     out.copy_(res)
     return out
 
 
-def moe_route_grouped(logits, top, groups, keep):
-    """Group-limited routing: (weights [T, top] fp32, ids [T, top] int32)."""
+def moe_route_grouped(logits, top, groups=1, keep=1, score="softmax",
+                      renorm=True, matrix=False):
+    """Group-limited routing: (weights [T, top] fp32, ids [T, top] int32);
+    score "softmax" or "sigmoid", renorm: the chosen scores divided by their
+    sum. matrix: also a [T, E] fp32 tensor holding each row's weights at
+    the experts it uses and 0 elsewhere."""
     if logits.is_cuda:
-        T = logits.shape[0]
+        T, E = logits.shape
         w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
         ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+        mat = (torch.empty((T, E), dtype=torch.float32, device=logits.device)
+               if matrix else None)
         _native_seq().moe_route_grouped(w, ids, logits.contiguous(), top,
-                                        groups, keep)
-        return w, ids
-    return ref.moe_route_grouped(logits, top, groups, keep)
+                                        groups, keep, score == "sigmoid",
+                                        bool(renorm), mat)
+        return (w, ids, mat) if matrix else (w, ids)
+    w, ids = ref.moe_route_grouped(logits, top, groups, keep, score, renorm)
+    if matrix:
+        return w, ids, ref.route_scale_matrix(w, ids, logits.shape[1])
+    return w, ids
 
 
 def moe_mix_seq(y, weights, ids):
@@ -1046,13 +1064,14 @@ def moe_mix_seq(y, weights, ids):
     return ref.moe_mix(y, weights, ids, 0)
 
 
-def moe_mix_rows_seq(y, weights, rows):
+def moe_mix_rows_seq(y, weights, rows, add=None):
+    """out[t] = sum_j weights[t, j] y[rows[t, j]] (+ add[t])."""
     if y.is_cuda:
         T, k = weights.shape
         out = torch.empty(T, y.shape[1], dtype=y.dtype, device=y.device)
-        _native_seq().moe_mix_rows(out, y.contiguous(), weights, rows)
+        _native_seq().moe_mix_rows(out, y.contiguous(), weights, rows, add)
         return out
-    return ref.moe_mix_rows(y, weights, rows)
+    return ref.moe_mix_rows(y, weights, rows, add)
 
 
 # ----------------------------------------------------------------------
@@ -1143,3 +1162,71 @@ def gate_group_norm(y, z, weight, groups, eps, out, out_scale=1.0):
                                       out_scale)
         return out
     return ref.gate_group_norm(y, z, weight, groups, eps, out, out_scale)
+
+
+# ----------------------------------------------------------------------
+# Two-norm parallel blocks with per-channel branch scales, difference
+# attention behind short convolutions, input-scaled experts (same
+# extension, same rule).
+# ----------------------------------------------------------------------
+def residual_pair_norm(x, y1, s1, y2, s2, w1, w2, eps, out_dtype):
+    """x (fp32 residual, in place) += s1 * y1 + s2 * y2 (each when given,
+    s per channel); returns (h1, h2), x divided by its root mean square
+    times (1 + w1) and (1 + w2), for each weight given — two norms of the
+    same rows from one pass."""
+    if x.is_cuda:
+        h1 = (torch.empty(x.shape, dtype=out_dtype, device=x.device)
+              if w1 is not None else None)
+        h2 = (torch.empty(x.shape, dtype=out_dtype, device=x.device)
+              if w2 is not None else None)
+        _native_seq().residual_pair_norm(x, h1, h2, y1, s1, y2, s2, w1, w2,
+                                         float(eps))
+        return h1, h2
+    return ref.residual_pair_norm(x, y1, s1, y2, s2, w1, w2, eps, out_dtype)
+
+
+def conv_qkv_cache(p, n_q, n_k, n_v, weight, weight_t, state, cu_seqlens,
+                   seq_lens, state_slots, token_seq, positions, temp_coef,
+                   temp_every, heads, kv_heads, maps, k_cache, v_cache,
+                   slot_mapping):
+    """Short causal convolution over the q | k | v channels of the
+    in-projection's rows, the position-dependent query factor, the query
+    heads regrouped by key map, keys and values to their pages, and the
+    sequences' new histories (ref.conv_qkv_cache). weight_t: [taps, C] copy
+    of the taps for the vectorised bf16 kernel. Returns q [T, n_q]."""
+    if p.is_cuda:
+        qo = torch.empty((p.shape[0], n_q), dtype=p.dtype, device=p.device)
+        _native_seq().conv_qkv_cache(
+            qo, p, n_q, n_k, n_v, weight, weight_t, state, cu_seqlens,
+            seq_lens, state_slots, token_seq, positions, float(temp_coef),
+            int(temp_every), heads, kv_heads, maps, k_cache, v_cache,
+            slot_mapping)
+        return qo
+    return ref.conv_qkv_cache(p, n_q, n_k, n_v, weight, state, cu_seqlens,
+                              seq_lens, state_slots, positions, temp_coef,
+                              temp_every, heads, kv_heads, maps, k_cache,
+                              v_cache, slot_mapping)
+
+
+def diff_head_norm_gate(a, gate, lam, eps, mult, heads, kv_heads, out):
+    """Two attention maps per head into one gated output row
+    (ref.diff_head_norm_gate): (a1 - lam a2) at unit RMS per head, times
+    mult, times sigmoid(gate)."""
+    if a.is_cuda:
+        _native_seq().diff_head_norm_gate(out, a, gate, float(lam), float(eps),
+                                          float(mult), heads, kv_heads)
+        return out
+    return ref.diff_head_norm_gate(a, gate, lam, eps, mult, heads, kv_heads,
+                                   out)
+
+
+def moe_glu_scaled(gu, scale, experts, ff, shared_ff):
+    """Activated rows of all experts side by side, each expert's gate and
+    up scaled by the row's weight for it, plus the shared expert's
+    (ref.moe_glu_scaled)."""
+    if gu.is_cuda:
+        out = torch.empty((gu.shape[0], experts * ff + shared_ff),
+                          dtype=gu.dtype, device=gu.device)
+        _native_seq().moe_glu_scaled(out, gu, scale, experts, ff, shared_ff)
+        return out
+    return ref.moe_glu_scaled(gu, scale, experts, ff, shared_ff)

@@ -289,11 +289,14 @@ def moe_mix(y: torch.Tensor, weights: torch.Tensor, ids: torch.Tensor,
 
 
 def moe_mix_rows(y: torch.Tensor, weights: torch.Tensor,
-                 rows: torch.Tensor) -> torch.Tensor:
-    """out[t] = sum_j weights[t,j] * y[rows[t,j]] over a flat [R, H]
-    expert-output buffer."""
+                 rows: torch.Tensor, add=None) -> torch.Tensor:
+    """out[t] = sum_j weights[t,j] * y[rows[t,j]] (+ add[t]) over a flat
+    [R, H] expert-output buffer."""
     gathered = y[rows.long()].float()  # [T, k, H]
-    return torch.einsum("tkh,tk->th", gathered, weights.float()).to(y.dtype)
+    out = torch.einsum("tkh,tk->th", gathered, weights.float())
+    if add is not None:
+        out = out + add.float()
+    return out.to(y.dtype)
 
 
 def quant_fp8_rows(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
@@ -401,26 +404,31 @@ def _rotate_pairs(x, angles, interleaved: bool):
 
 def qk_norm_rope_cache(q, k, v, q_norm_w, k_norm_w, eps, positions,
                        inv_freq_qk, inv_freq_v, k_cache, v_cache,
-                       slot_mapping, interleaved=True):
+                       slot_mapping, interleaved=True, rot_mag=1.0,
+                       unit_norm_after=False):
     """q [T,H,D], k [T,G,D], v [T,G,V]: per-head RMS norm of q and k (weights
-    or None), rotary on their first 2*len(inv_freq_qk) dims, values turned by
+    or None), rotary on their first 2*len(inv_freq_qk) dims with cos and sin
+    times rot_mag, then (unit_norm_after) q and k divided by their root mean
+    square over the head once more, without a weight; values turned by
     their own position over all V dims (inv_freq_v None = values stored
     plain); k and v go to the paged cache. Returns q (fp32 math, q.dtype)."""
     pos = positions.float()
 
-    def prep(t, w, inv_freq):
+    def prep(t, w, inv_freq, mag=1.0, after=False):
         tf = t.float()
         if w is not None:
             tf = tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
         if inv_freq is not None and inv_freq.numel():
             rd = 2 * inv_freq.numel()
             ang = pos[:, None, None] * inv_freq.float()[None, None, :]
-            tf = torch.cat([_rotate_pairs(tf[..., :rd], ang, interleaved),
+            tf = torch.cat([_rotate_pairs(tf[..., :rd], ang, interleaved) * mag,
                             tf[..., rd:]], -1)
+        if after:
+            tf = tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + eps)
         return tf
 
-    qo = prep(q, q_norm_w, inv_freq_qk).to(q.dtype)
-    ko = prep(k, k_norm_w, inv_freq_qk).to(k_cache.dtype)
+    qo = prep(q, q_norm_w, inv_freq_qk, rot_mag, unit_norm_after).to(q.dtype)
+    ko = prep(k, k_norm_w, inv_freq_qk, rot_mag, unit_norm_after).to(k_cache.dtype)
     vo = prep(v, None, inv_freq_v).to(v_cache.dtype)
     bs = k_cache.shape[2]
     ok = slot_mapping >= 0
@@ -434,8 +442,11 @@ def qk_norm_rope_cache(q, k, v, q_norm_w, k_norm_w, eps, positions,
 def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
                          cu_seqlens, scale, sink=True, inv_freq_v=None,
                          interleaved=True, sink_w=None, softcap=0.0,
-                         window=0, keep_first=0):
+                         window=0, keep_first=0, maps=1):
     """Causal attention of packed new rows over each sequence's paged keys.
+    maps M > 1: a key row holds M keys of D dims side by side (k_cache
+    [pages, G, bs, M*D]) that share the row's value; q has G*M groups of
+    query heads, group g*M + m reads key m of key/value head g.
     sink=True adds a value-less key of score 0 to every softmax (one more
     in the denominator); sink_w [H] gives that key a score per head
     instead (taken as it is: neither scaled nor capped). softcap c > 0:
@@ -455,10 +466,13 @@ def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
             continue
         nb = (L + bs - 1) // bs
         pages = block_tables[s, :nb].long()
-        K = k_cache[pages].permute(1, 0, 2, 3).reshape(G, nb * bs, D)[:, :L].float()
+        K = k_cache[pages].permute(1, 0, 2, 3).reshape(G, nb * bs, maps * D)[:, :L].float()
         Vv = v_cache[pages].permute(1, 0, 2, 3).reshape(G, nb * bs, V)[:, :L].float()
-        K = K.repeat_interleave(H // G, 0)
-        Vv = Vv.repeat_interleave(H // G, 0)
+        if maps > 1:
+            K = K.view(G, L, maps, D).transpose(1, 2).reshape(G * maps, L, D)
+            Vv = Vv.repeat_interleave(maps, 0)
+        K = K.repeat_interleave(H // (G * maps), 0)
+        Vv = Vv.repeat_interleave(H // (G * maps), 0)
         qs = q[a:b].float().permute(1, 0, 2)  # [H, n, D]
         sc = torch.matmul(qs, K.transpose(1, 2)) * scale  # [H, n, L]
         qpos = torch.arange(L - n, L)
@@ -747,14 +761,17 @@ def head_norm_gate(o, gate, eps, heads, out, out_scale=1.0):
     return out
 
 
-def glu_act(gu, kind, limit=0.0, alpha=1.0):
-    """gu [T, 2F] = [gate | up] -> [T, F].
+def glu_act(gu, kind, limit=0.0, alpha=1.0, row_scale=None):
+    """gu [T, 2F] = [gate | up] -> [T, F]; row_scale [T] fp32 multiplies a
+    row's gate and up first (the projections of a scaled input).
     "swiglu": silu(gate) * up.
     "clamped": g = min(gate, limit), u = clamp(up, -limit, limit),
                g * sigmoid(alpha g) * (u + 1).
     "gelu_tanh": gelu_tanh(gate) * up."""
     F_ = gu.shape[-1] // 2
     g, u = gu[..., :F_].float(), gu[..., F_:].float()
+    if row_scale is not None:
+        g, u = g * row_scale.float()[:, None], u * row_scale.float()[:, None]
     if kind == "swiglu":
         return (g * torch.sigmoid(g) * u).to(gu.dtype)
     if kind == "gelu_tanh":
@@ -764,13 +781,17 @@ def glu_act(gu, kind, limit=0.0, alpha=1.0):
     return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
 
 
-def moe_route_grouped(logits, top, groups, keep):
-    """Softmax over all experts; experts are cut into `groups`
+def moe_route_grouped(logits, top, groups, keep, score="softmax",
+                      renorm=True):
+    """Scores over all experts: their softmax, or (score="sigmoid") each
+    logit's own sigmoid; without renorm the chosen scores are the weights as
+    they are. Experts are cut into `groups`
     contiguous runs of E/groups, a run's score is its highest expert score
     and only the `keep` highest-scoring runs stay eligible; the `top` largest scores among those, their
     scores divided by their sum (+1e-20). Ties go to the lower index.
     logits [T, E] fp32 -> (weights [T, top] fp32, ids [T, top] int32)."""
-    s = torch.softmax(logits.float(), -1)
+    s = (torch.sigmoid(logits.float()) if score == "sigmoid"
+         else torch.softmax(logits.float(), -1))
     T, E = s.shape
     per = E // groups
     gs = s.view(T, groups, per).amax(-1)
@@ -781,7 +802,8 @@ def moe_route_grouped(logits, top, groups, keep):
                          s, torch.full_like(s, -1.0))
     ids = torch.topk(masked, top, dim=-1).indices
     w = s.gather(1, ids)
-    w = w / (w.sum(-1, keepdim=True) + 1e-20)
+    if renorm:
+        w = w / (w.sum(-1, keepdim=True) + 1e-20)
     return w, ids.to(torch.int32)
 
 
@@ -876,4 +898,122 @@ def gate_group_norm(y, z, weight, groups, eps, out, out_scale=1.0):
     g = g.view(T, groups, C // groups)
     g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)
     out.copy_((g.reshape(T, C) * weight.float() * out_scale).to(out.dtype))
+    return out
+
+
+# ----------------------------------------------------------------------
+# Two-norm parallel blocks with per-channel branch scales, difference
+# attention behind short convolutions, input-scaled experts.
+# ----------------------------------------------------------------------
+def residual_pair_norm(x, y1, s1, y2, s2, w1, w2, eps, out_dtype):
+    """x (fp32, in place) += s1 * y1 + s2 * y2 (each when given; s per
+    channel); returns (h1, h2) = x / sqrt(mean(x^2) + eps) * (1 + w) for
+    each weight given (None otherwise), in out_dtype."""
+    if y1 is not None:
+        add = y1.float() * s1.float()
+        if y2 is not None:
+            add = add + y2.float() * s2.float()
+        x += add
+    elif y2 is not None:
+        x += y2.float() * s2.float()
+    if w1 is None and w2 is None:
+        return None, None
+    n = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    return tuple((n * (1.0 + w.float())).to(out_dtype) if w is not None
+                 else None for w in (w1, w2))
+
+
+def query_map_order(c, heads, kv_heads, maps, dim):
+    """Where channel c of a query row laid out [head, map, dim] goes in the
+    order [kv head, map, head of the group, dim] the attention ops read."""
+    d = c % dim
+    m = (c // dim) % maps
+    h = c // (dim * maps)
+    r = heads // kv_heads
+    return (((h // r) * maps + m) * r + h % r) * dim + d
+
+
+def conv_qkv_cache(p, n_q, n_k, n_v, weight, state, cu_seqlens, seq_lens,
+                   state_slots, positions, temp_coef, temp_every, heads,
+                   kv_heads, maps, k_cache, v_cache, slot_mapping):
+    """Causal depthwise convolution over time of the first n_q + n_k + n_v
+    channels of p [T, >=C] (weight [C, taps], last column = current row, no
+    bias, no activation; state [slots, taps-1, C] fp32 holds each sequence's
+    last taps-1 inputs and is updated). The q channels are multiplied by
+    1 + temp_coef ln(floor((pos + 1) / temp_every) + 1) (temp_every 0: by 1)
+    and returned [T, n_q] in the head order of query_map_order; the k and v
+    channels go to their pages (k_cache [pages, G, bs, n_k / G])."""
+    T = p.shape[0]
+    C = n_q + n_k + n_v
+    taps = weight.shape[1]
+    xf = p[:, :C].float()
+    y = torch.empty(T, C, dtype=torch.float32)
+    wf = weight.float()
+    for a, b, start, slot in _seq_spans(cu_seqlens, seq_lens, state_slots):
+        hist = (state[slot].clone() if start > 0 and slot >= 0 and taps > 1
+                else torch.zeros(taps - 1, C))
+        full = torch.cat([hist, xf[a:b]], 0)
+        n = b - a
+        acc = torch.zeros(n, C)
+        for j in range(taps):
+            acc += full[j:j + n] * wf[:, j][None, :]
+        y[a:b] = acc
+        if slot >= 0 and taps > 1:
+            state[slot] = full[n:]
+    q = y[:, :n_q]
+    if temp_every > 0:
+        pos = positions.float()
+        q = q * (1.0 + temp_coef * torch.log(
+            torch.floor((pos + 1.0) / temp_every) + 1.0))[:, None]
+    dim = n_q // (heads * maps)
+    order = query_map_order(torch.arange(n_q), heads, kv_heads, maps, dim)
+    qo = torch.empty(T, n_q, dtype=p.dtype)
+    qo[:, order] = q.to(p.dtype)
+    if n_k:
+        G, bs = k_cache.shape[1], k_cache.shape[2]
+        ok = slot_mapping >= 0
+        blk = (slot_mapping[ok] // bs).long()
+        off = (slot_mapping[ok] % bs).long()
+        k_cache[blk, :, off] = y[ok, n_q:n_q + n_k].view(-1, G, n_k // G).to(k_cache.dtype)
+        v_cache[blk, :, off] = y[ok, n_q + n_k:].view(-1, G, n_v // G).to(v_cache.dtype)
+    return qo
+
+
+def diff_head_norm_gate(a, gate, lam, eps, mult, heads, kv_heads, out):
+    """a [T, kv_heads, 2, heads / kv_heads, V]: the two maps' outputs of
+    every head. o = a[:, :, 0] - lam * a[:, :, 1], divided by its root mean
+    square over V, times mult, times sigmoid(gate) (gate [T, heads * V] in
+    the plain head order), into out [T, heads * V] (views, any row
+    stride)."""
+    T = a.shape[0]
+    V = a.shape[-1]
+    af = a.float().view(T, kv_heads, 2, heads // kv_heads, V)
+    o = (af[:, :, 0] - lam * af[:, :, 1]).reshape(T, heads, V)
+    o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * mult
+    out.copy_((o.reshape(T, heads * V) * torch.sigmoid(gate.float())).to(out.dtype))
+    return out
+
+
+def moe_glu_scaled(gu, scale, experts, ff, shared_ff):
+    """gu [T, experts * 2 ff + 2 shared_ff]: per expert [gate | up], then
+    the shared expert's [gate | up]. Column c of expert e becomes
+    silu(s g) * (s u) with s = scale[t, e] (fp32; 0 for an expert the row
+    does not use), the shared columns silu(g) * u. -> [T, experts * ff +
+    shared_ff]."""
+    T = gu.shape[0]
+    ex = gu[:, :experts * 2 * ff].float().view(T, experts, 2, ff)
+    s = scale.float()[:, :, None]
+    g, u = ex[:, :, 0] * s, ex[:, :, 1] * s
+    parts = [(g * torch.sigmoid(g) * u).reshape(T, experts * ff)]
+    if shared_ff:
+        sh = gu[:, experts * 2 * ff:].float()
+        g, u = sh[:, :shared_ff], sh[:, shared_ff:]
+        parts.append(g * torch.sigmoid(g) * u)
+    return torch.cat(parts, -1).to(gu.dtype)
+
+
+def route_scale_matrix(weights, ids, experts):
+    """[T, experts] fp32: a row's weight at each expert it uses, 0 elsewhere."""
+    out = torch.zeros(weights.shape[0], experts, dtype=torch.float32)
+    out.scatter_(1, ids.long(), weights.float())
     return out
