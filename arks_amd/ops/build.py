@@ -55,6 +55,7 @@ SEQ_SOURCES = [
     os.path.join(CSRC, "seq_shared.hip"),
     os.path.join(CSRC, "seq_mamba2.hip"),
     os.path.join(CSRC, "seq_masked_mfma.hip"),
+    os.path.join(CSRC, "seq_dual.hip"),
 ]
 
 EXTENSIONS = {EXT_NAME: SOURCES, SEQ_EXT_NAME: SEQ_SOURCES}

@@ -16,7 +16,10 @@
 // value may be a leading part of the key's row (latent attention keeps one
 // row per token for both). The output is a row-strided view (ldo), scaled
 // by out_scale. After the sum each row's output is turned back by its own
-// position when the cache holds position-turned values.
+// position when the cache holds position-turned values. maps M > 1: a key
+// row holds M keys of D dims side by side (row stride ldk >= M * D) that
+// share the row's value; H counts all query heads, in H / (G * M)-head
+// groups, and group g * M + m reads key m of key/value head g.
 #include "seq_common.h"
 
 namespace arks {
@@ -33,7 +36,8 @@ __global__ __launch_bounds__(64) void attn_sink_generic_kernel(
     float scale, int sink, const float* __restrict__ freq_v, int interleaved,
     int H, int G, int D, int V, int block_size, int max_blocks,
     const float* __restrict__ sink_w, float softcap, int window,
-    int keep_first, int64_t ldk, int64_t ldv, int64_t ldo, float out_scale) {
+    int keep_first, int64_t ldk, int64_t ldv, int64_t ldo, float out_scale,
+    int maps) {
   __shared__ float q_s[ATT_MAX_D];
   __shared__ float p_s[64];
   __shared__ int64_t voff_s[64];
@@ -44,7 +48,9 @@ __global__ __launch_bounds__(64) void attn_sink_generic_kernel(
   const int rows = cu[s + 1] - first_row;
   const int pos = seq_lens[s] - rows + (t - first_row);
   const int nkeys = pos + 1;
-  const int g = h / (H / G);
+  const int gm = h / (H / (G * maps));  // key group: (kv head, map)
+  const int g = gm / maps;
+  const int kcol = (gm % maps) * D;
   const int* bt = block_tables + (int64_t)s * max_blocks;
   for (int d = lane; d < D; d += 64)
     q_s[d] = Act<AT>::ld(q + ((int64_t)t * H + h) * D + d);
@@ -65,7 +71,7 @@ __global__ __launch_bounds__(64) void attn_sink_generic_kernel(
     if (valid) {
       const int page = bt[j / block_size];
       rowoff = ((int64_t)page * G + g) * block_size + (j % block_size);
-      const AT* kr = k_cache + rowoff * ldk;
+      const AT* kr = k_cache + rowoff * ldk + kcol;
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot += q_s[d] * Act<AT>::ld(kr + d);
       sc = dot * scale;
@@ -134,7 +140,7 @@ extern "C" int arks_seq_attn_sink_generic(
     int interleaved, int T, int H, int G, int D, int V, int block_size,
     int max_blocks, int act_f32, const void* sink_w, float softcap,
     int window, int keep_first, int64_t ldk, int64_t ldv, int64_t ldo,
-    float out_scale, hipStream_t stream) {
+    float out_scale, int maps, hipStream_t stream) {
   if (D > ATT_MAX_D || V > 64 * ATT_VPT) return 1;
   if (T == 0) return 0;
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
@@ -143,6 +149,6 @@ extern "C" int arks_seq_attn_sink_generic(
       (const int*)block_tables, (const int*)seq_lens, (const int*)cu,
       (const int*)token_seq, scale, sink, (const float*)freq_v, interleaved, H,
       G, D, V, block_size, max_blocks, (const float*)sink_w, softcap, window,
-      keep_first, ldk, ldv, ldo, out_scale));
+      keep_first, ldk, ldv, ldo, out_scale, maps));
   return 0;
 }

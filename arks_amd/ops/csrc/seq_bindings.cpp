@@ -27,7 +27,7 @@ int arks_seq_qk_norm_rope_cache(
     const void* positions, const void* freq_qk, int n_rot, const void* freq_v,
     int n_vrot, void* k_cache, void* v_cache, const void* slot_mapping, int T,
     int H, int G, int D, int V, int block_size, int interleaved, int act_f32,
-    hipStream_t stream);
+    float rot_mag, int norm_after, hipStream_t stream);
 int arks_seq_unrotate_rows(void* out, const void* positions, const void* freq,
                             int T, int H, int V, int interleaved, int act_f32,
                             hipStream_t stream);
@@ -38,7 +38,7 @@ int arks_seq_attn_sink_generic(
     int interleaved, int T, int H, int G, int D, int V, int block_size,
     int max_blocks, int act_f32, const void* sink_w, float softcap,
     int window, int keep_first, int64_t ldk, int64_t ldv, int64_t ldo,
-    float out_scale, hipStream_t stream);
+    float out_scale, int maps, hipStream_t stream);
 int arks_seq_lightning_scan(void* out, const void* q, const void* k,
                             const void* v, int64_t ldq, int64_t ldk,
                             int64_t ldv, const void* decay, void* state,
@@ -89,7 +89,7 @@ void arks_seq_head_norm_gate(void* out, int64_t ldo, const void* o,
                              hipStream_t stream);
 void arks_seq_glu_act(void* out, int64_t ldo, const void* gu, int64_t ldg,
                       int64_t rows, int F, int mode, float limit, float alpha,
-                      int act_f32, hipStream_t stream);
+                      const void* row_scale, int act_f32, hipStream_t stream);
 void arks_seq_kv_write_pooled(const void* k, const void* v, int64_t ldk,
                               int64_t ldv, void* k_cache, void* v_cache,
                               void* kp_cache, void* vp_cache,
@@ -162,10 +162,33 @@ int arks_seq_attn_masked_mfma(void* out, int64_t ldo, const void* q,
 int arks_seq_attn_masked_ksplit(int T, int H, int G, int max_blocks);
 int arks_seq_moe_route_grouped(void* weights, void* ids, const void* logits,
                                int T, int E, int top, int groups, int keep,
+                               int sigmoid, int renorm, void* matrix,
                                hipStream_t stream);
 void arks_seq_moe_mix_rows(void* out, const void* y, const void* weights,
                            const void* rows, int T, int H, int k, int dense,
-                           int act_f32, hipStream_t stream);
+                           const void* add, int act_f32, hipStream_t stream);
+void arks_seq_residual_pair_norm(void* x, void* h1, void* h2, const void* y1,
+                                 const void* s1, const void* y2,
+                                 const void* s2, const void* w1,
+                                 const void* w2, float eps, int64_t T, int C,
+                                 int act_f32, hipStream_t stream);
+int arks_seq_conv_qkv_cache(void* qo, const void* p, int64_t ldp,
+                            const void* w, const void* w_t, void* state,
+                            const void* cu, const void* seq_lens,
+                            const void* slots, const void* token_seq,
+                            const void* positions, void* k_cache,
+                            void* v_cache, const void* slot_mapping, int T,
+                            int S, int n_q, int n_k, int n_v, int heads,
+                            int kv_heads, int maps, int block_size, int taps,
+                            float temp_coef, int temp_every, int act_f32,
+                            hipStream_t stream);
+int arks_seq_diff_head_norm_gate(void* out, int64_t ldo, const void* a,
+                                 const void* gate, int64_t ldg, float lam,
+                                 float eps, float mult, int T, int H, int G,
+                                 int V, int act_f32, hipStream_t stream);
+void arks_seq_moe_glu_scaled(void* out, const void* gu, int64_t ldg,
+                             const void* scale, int64_t T, int E, int ff,
+                             int sff, int act_f32, hipStream_t stream);
 void arks_seq_lightning_combine(void* part, const void* decay, void* state,
                                 const void* chunk_off, const void* chunk_rows,
                                 const void* cu, const void* seq_lens,
@@ -343,7 +366,8 @@ void gelu_tanh(Tensor out, Tensor x) {
 void qk_norm_rope_cache(Tensor qo, Tensor q, Tensor k, Tensor v, OptTensor qw,
                         OptTensor kw, double eps, Tensor positions,
                         Tensor freq_qk, OptTensor freq_v, Tensor k_cache,
-                        Tensor v_cache, Tensor slot_mapping, bool interleaved) {
+                        Tensor v_cache, Tensor slot_mapping, bool interleaved,
+                        double rot_mag, bool norm_after) {
   const int f32 = act_flag(q, "q");
   const int T = q.size(0), H = q.size(1), D = q.size(2);
   const int G = k.size(1), V = v.size(2);
@@ -392,7 +416,8 @@ void qk_norm_rope_cache(Tensor qo, Tensor q, Tensor k, Tensor v, OptTensor qw,
       qw_p, kw_p, (float)eps, positions.data_ptr(), freq_qk.data_ptr(), n_rot,
       fv_p, n_vrot, k_cache.data_ptr(), v_cache.data_ptr(),
       slot_mapping.data_ptr(), T, H, G, D, V, (int)k_cache.size(2),
-      interleaved ? 1 : 0, f32, current_stream());
+      interleaved ? 1 : 0, f32, (float)rot_mag, norm_after ? 1 : 0,
+      current_stream());
   TORCH_CHECK(rc == 0, "more rotary pairs than the kernel's table holds");
 }
 
@@ -402,16 +427,20 @@ void attention_sink_paged(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
                           OptTensor freq_v, bool interleaved,
                           int64_t max_q_len, OptTensor sink_w, double softcap,
                           int64_t window, int64_t keep_first,
-                          double out_scale) {
+                          double out_scale, int64_t maps) {
   const int f32 = act_flag(q, "q");
-  TORCH_CHECK(q.is_contiguous() && q.dim() == 3);
+  TORCH_CHECK(q.is_contiguous() && q.dim() == 3 && maps >= 1);
   const int T = q.size(0), H = q.size(1), D = q.size(2);
   TORCH_CHECK(k_cache.scalar_type() == q.scalar_type() &&
               v_cache.scalar_type() == q.scalar_type() &&
               out.scalar_type() == q.scalar_type());
-  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(3) == D);
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 &&
+              k_cache.size(3) == D * maps);
   const int G = k_cache.size(1), bs = k_cache.size(2), V = v_cache.size(3);
-  TORCH_CHECK(H % G == 0 && v_cache.size(1) == G && v_cache.size(2) == bs);
+  TORCH_CHECK(H % (G * maps) == 0 && v_cache.size(1) == G &&
+              v_cache.size(2) == bs);
+  TORCH_CHECK(maps == 1 || (!sink_w.has_value() && !freq_v.has_value()),
+              "several key maps: no per-head sink, no turned values");
   const int64_t ldk = paged_row_stride(k_cache, "k_cache");
   const int64_t ldv = paged_row_stride(v_cache, "v_cache");
   const int64_t ldo = head_row_stride(out, "out");
@@ -439,7 +468,7 @@ void attention_sink_paged(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
       token_seq.data_ptr(), (float)scale, sink ? 1 : 0, fv_p,
       interleaved ? 1 : 0, T, H, G, D, V, bs, (int)block_tables.size(1), f32,
       sw_p, (float)softcap, (int)window, (int)keep_first, ldk, ldv, ldo,
-      (float)out_scale, current_stream());
+      (float)out_scale, (int)maps, current_stream());
   TORCH_CHECK(rc == 0, "attention head sizes beyond the kernel's limits (",
               D, ", ", V, ")");
 }
@@ -760,15 +789,22 @@ void head_norm_gate(Tensor out, Tensor o, Tensor gate, double eps,
                           (float)out_scale, f32, current_stream());
 }
 
-void glu_act(Tensor out, Tensor gu, int64_t mode, double limit, double alpha) {
+void glu_act(Tensor out, Tensor gu, int64_t mode, double limit, double alpha,
+             OptTensor row_scale) {
   const int f32 = act_flag(gu, "gate|up");
   TORCH_CHECK(gu.dim() == 2 && gu.size(1) % 2 == 0);
   const int F = gu.size(1) / 2;
   TORCH_CHECK(out.scalar_type() == gu.scalar_type() &&
               out.size(0) == gu.size(0) && out.size(1) == F);
+  const void* rs_p = nullptr;
+  if (row_scale.has_value()) {
+    check_f32(*row_scale, "row_scale");
+    TORCH_CHECK(row_scale->numel() == gu.size(0));
+    rs_p = row_scale->data_ptr();
+  }
   arks_seq_glu_act(out.data_ptr(), row_stride(out, "out"), gu.data_ptr(),
                    row_stride(gu, "gate|up"), gu.size(0), F, (int)mode,
-                   (float)limit, (float)alpha, f32, current_stream());
+                   (float)limit, (float)alpha, rs_p, f32, current_stream());
 }
 
 struct WindowShapes {
@@ -885,21 +921,30 @@ bool attention_window_pool_mfma(Tensor out, Tensor q, Tensor k_cache,
 }
 
 void moe_route_grouped(Tensor weights, Tensor ids, Tensor logits, int64_t top,
-                       int64_t groups, int64_t keep) {
+                       int64_t groups, int64_t keep, bool sigmoid, bool renorm,
+                       OptTensor matrix) {
   check_f32(logits, "router logits");
   check_f32(weights, "weights");
   check_i32(ids, "ids");
   const int T = logits.size(0), E = logits.size(1);
   TORCH_CHECK(weights.size(0) == T && weights.size(1) == top &&
               ids.size(0) == T && ids.size(1) == top);
+  void* mat_p = nullptr;
+  if (matrix.has_value()) {
+    check_f32(*matrix, "scale matrix");
+    TORCH_CHECK(matrix->dim() == 2 && matrix->size(0) == T &&
+                matrix->size(1) == E);
+    mat_p = matrix->data_ptr();
+  }
   const int rc = arks_seq_moe_route_grouped(
       weights.data_ptr(), ids.data_ptr(), logits.data_ptr(), T, E, (int)top,
-      (int)groups, (int)keep, current_stream());
+      (int)groups, (int)keep, sigmoid ? 1 : 0, renorm ? 1 : 0, mat_p,
+      current_stream());
   TORCH_CHECK(rc == 0, "routing sizes the kernel does not hold");
 }
 
 void moe_mix_common(Tensor out, Tensor y, Tensor weights, Tensor rows,
-                    int dense) {
+                    int dense, const OptTensor& add = c10::nullopt) {
   const int f32 = act_flag(y, "y");
   check_f32(weights, "weights");
   check_i32(rows, "rows");
@@ -909,16 +954,163 @@ void moe_mix_common(Tensor out, Tensor y, Tensor weights, Tensor rows,
   TORCH_CHECK(out.size(0) == T && rows.numel() == (int64_t)T * k &&
               y.size(-1) == H);
   if (dense) TORCH_CHECK(y.dim() == 3 && y.size(1) == T);
+  const void* add_p = nullptr;
+  if (add.has_value()) {
+    TORCH_CHECK(add->scalar_type() == y.scalar_type() && add->is_contiguous() &&
+                add->is_cuda() && add->sizes() == out.sizes());
+    add_p = add->data_ptr();
+  }
   arks_seq_moe_mix_rows(out.data_ptr(), y.data_ptr(), weights.data_ptr(),
-                        rows.data_ptr(), T, H, k, dense, f32, current_stream());
+                        rows.data_ptr(), T, H, k, dense, add_p, f32,
+                        current_stream());
 }
 
 void moe_mix(Tensor out, Tensor y, Tensor weights, Tensor ids) {
   moe_mix_common(out, y, weights, ids, 1);
 }
 
-void moe_mix_rows(Tensor out, Tensor y, Tensor weights, Tensor rows) {
-  moe_mix_common(out, y, weights, rows, 0);
+void moe_mix_rows(Tensor out, Tensor y, Tensor weights, Tensor rows,
+                  OptTensor add) {
+  moe_mix_common(out, y, weights, rows, 0, add);
+}
+
+void residual_pair_norm(Tensor x, OptTensor h1, OptTensor h2, OptTensor y1,
+                        OptTensor s1, OptTensor y2, OptTensor s2, OptTensor w1,
+                        OptTensor w2, double eps) {
+  check_f32(x, "x");
+  TORCH_CHECK(x.dim() == 2);
+  const int64_t T = x.size(0);
+  const int C = x.size(1);
+  int f32 = -1;
+  auto rows = [&](const OptTensor& t, const char* name) -> void* {
+    if (!t.has_value()) return nullptr;
+    const int f = act_flag(*t, name);
+    TORCH_CHECK(f32 < 0 || f == f32, "activation dtypes differ");
+    f32 = f;
+    TORCH_CHECK(t->dim() == 2 && t->size(0) == T && t->size(1) == C &&
+                t->is_contiguous(), name, " must be contiguous [T, C]");
+    return t->data_ptr();
+  };
+  auto vec = [&](const OptTensor& t, const char* name) -> const void* {
+    if (!t.has_value()) return nullptr;
+    check_f32(*t, name);
+    TORCH_CHECK(t->numel() == C, name, " must have C entries");
+    return t->data_ptr();
+  };
+  void* h1_p = rows(h1, "h1");
+  void* h2_p = rows(h2, "h2");
+  const void* y1_p = rows(y1, "y1");
+  const void* y2_p = rows(y2, "y2");
+  TORCH_CHECK(h1.has_value() == w1.has_value() &&
+              h2.has_value() == w2.has_value() &&
+              y1.has_value() == s1.has_value() &&
+              y2.has_value() == s2.has_value());
+  if (f32 < 0) return;  // nothing to add, nothing to write
+  arks_seq_residual_pair_norm(x.data_ptr(), h1_p, h2_p, y1_p, vec(s1, "s1"),
+                              y2_p, vec(s2, "s2"), vec(w1, "w1"),
+                              vec(w2, "w2"), (float)eps, T, C, f32,
+                              current_stream());
+}
+
+void conv_qkv_cache(Tensor qo, Tensor p, int64_t n_q, int64_t n_k, int64_t n_v,
+                    Tensor w, OptTensor w_t, OptTensor state, Tensor cu,
+                    Tensor seq_lens, Tensor slots, Tensor token_seq,
+                    Tensor positions, double temp_coef, int64_t temp_every,
+                    int64_t heads, int64_t kv_heads, int64_t maps,
+                    OptTensor k_cache, OptTensor v_cache, Tensor slot_mapping) {
+  const int f32 = act_flag(p, "p");
+  const int64_t ldp = row_stride(p, "p");
+  const int T = p.size(0);
+  const int64_t C = n_q + n_k + n_v;
+  TORCH_CHECK(p.size(1) >= C && n_q > 0 && heads > 0 && kv_heads > 0 &&
+              maps > 0 && heads % kv_heads == 0 &&
+              n_q % (heads * maps) == 0 && n_k % kv_heads == 0 &&
+              n_v % kv_heads == 0);
+  TORCH_CHECK(qo.scalar_type() == p.scalar_type() && qo.is_contiguous() &&
+              qo.dim() == 2 && qo.size(0) == T && qo.size(1) == n_q);
+  check_f32(w, "taps");
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == C);
+  const int taps = w.size(1);
+  const void* wt_p = nullptr;
+  if (w_t.has_value()) {
+    check_f32(*w_t, "transposed taps");
+    TORCH_CHECK(w_t->dim() == 2 && w_t->size(0) == taps && w_t->size(1) == C);
+    wt_p = w_t->data_ptr();
+  }
+  const SeqMeta m = check_meta(cu, seq_lens, &slots, &token_seq, T);
+  void* st_p = nullptr;
+  if (taps > 1) {
+    TORCH_CHECK(state.has_value(), "a convolution with history needs state");
+    check_f32(*state, "conv state");
+    TORCH_CHECK(state->dim() == 3 && state->size(1) == taps - 1 &&
+                state->size(2) == C);
+    st_p = state->data_ptr();
+  }
+  check_i64(positions, "positions");
+  check_i64(slot_mapping, "slot_mapping");
+  TORCH_CHECK(positions.numel() == T && slot_mapping.numel() == T);
+  void* kc_p = nullptr;
+  void* vc_p = nullptr;
+  int bs = 1;
+  if (n_k > 0 || n_v > 0) {
+    TORCH_CHECK(k_cache.has_value() && v_cache.has_value());
+    TORCH_CHECK(k_cache->scalar_type() == p.scalar_type() &&
+                v_cache->scalar_type() == p.scalar_type() &&
+                k_cache->is_contiguous() && v_cache->is_contiguous() &&
+                k_cache->dim() == 4 && v_cache->dim() == 4);
+    TORCH_CHECK(k_cache->size(1) == kv_heads && v_cache->size(1) == kv_heads &&
+                k_cache->size(3) * kv_heads == n_k &&
+                v_cache->size(3) * kv_heads == n_v &&
+                k_cache->size(2) == v_cache->size(2) &&
+                k_cache->size(0) == v_cache->size(0), "cache shape mismatch");
+    kc_p = k_cache->data_ptr();
+    vc_p = v_cache->data_ptr();
+    bs = k_cache->size(2);
+  }
+  const int rc = arks_seq_conv_qkv_cache(
+      qo.data_ptr(), p.data_ptr(), ldp, w.data_ptr(), wt_p, st_p,
+      cu.data_ptr(), seq_lens.data_ptr(), slots.data_ptr(),
+      token_seq.data_ptr(), positions.data_ptr(), kc_p, vc_p,
+      slot_mapping.data_ptr(), T, m.S, (int)n_q, (int)n_k, (int)n_v,
+      (int)heads, (int)kv_heads, (int)maps, bs, taps, (float)temp_coef,
+      (int)temp_every, f32, current_stream());
+  TORCH_CHECK(rc == 0, "more taps than the convolution kernel holds");
+}
+
+void diff_head_norm_gate(Tensor out, Tensor a, Tensor gate, double lam,
+                         double eps, double mult, int64_t heads,
+                         int64_t kv_heads) {
+  const int f32 = act_flag(a, "a");
+  TORCH_CHECK(a.is_contiguous() && a.dim() == 3 && a.size(1) == 2 * heads &&
+              heads % kv_heads == 0);
+  const int T = a.size(0), V = a.size(2);
+  TORCH_CHECK(out.scalar_type() == a.scalar_type() &&
+              gate.scalar_type() == a.scalar_type() && out.dim() == 2 &&
+              gate.dim() == 2 && out.size(0) == T && gate.size(0) == T &&
+              out.size(1) == heads * V && gate.size(1) == heads * V);
+  const int rc = arks_seq_diff_head_norm_gate(
+      out.data_ptr(), row_stride(out, "out"), a.data_ptr(), gate.data_ptr(),
+      row_stride(gate, "gate"), (float)lam, (float)eps, (float)mult, T,
+      (int)heads, (int)kv_heads, V, f32, current_stream());
+  TORCH_CHECK(rc == 0, "value size beyond the kernel's limit (", V, ")");
+}
+
+void moe_glu_scaled(Tensor out, Tensor gu, Tensor scale, int64_t experts,
+                    int64_t ff, int64_t shared_ff) {
+  const int f32 = act_flag(gu, "gate|up");
+  check_f32(scale, "scale");
+  const int64_t T = gu.size(0);
+  TORCH_CHECK(gu.dim() == 2 &&
+              gu.size(1) == experts * 2 * ff + 2 * shared_ff &&
+              scale.dim() == 2 && scale.size(0) == T &&
+              scale.size(1) == experts);
+  TORCH_CHECK(out.scalar_type() == gu.scalar_type() && out.is_contiguous() &&
+              out.dim() == 2 && out.size(0) == T &&
+              out.size(1) == experts * ff + shared_ff);
+  arks_seq_moe_glu_scaled(out.data_ptr(), gu.data_ptr(),
+                          row_stride(gu, "gate|up"), scale.data_ptr(), T,
+                          (int)experts, (int)ff, (int)shared_ff, f32,
+                          current_stream());
 }
 
 }  // namespace
@@ -1104,7 +1296,8 @@ bool attention_masked_mfma(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
                            Tensor block_tables, Tensor seq_lens, Tensor cu,
                            Tensor token_seq, double scale, OptTensor sink_w,
                            double softcap, int64_t window, int64_t keep_first,
-                           double out_scale, bool single_rows) {
+                           double out_scale, bool single_rows, int64_t maps) {
+  if (maps != 1) return false;
   TORCH_CHECK(q.is_cuda() && q.scalar_type() == torch::kBFloat16 &&
               q.is_contiguous() && q.dim() == 3);
   const int T = q.size(0), H = q.size(1), D = q.size(2);
@@ -1154,6 +1347,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("mamba2_scan", &mamba2_scan);
   m.def("mamba2_combine", &mamba2_combine);
   m.def("gate_group_norm", &gate_group_norm);
+  m.def("residual_pair_norm", &residual_pair_norm);
+  m.def("conv_qkv_cache", &conv_qkv_cache);
+  m.def("diff_head_norm_gate", &diff_head_norm_gate);
+  m.def("moe_glu_scaled", &moe_glu_scaled);
   m.def("attention_masked_mfma", &attention_masked_mfma);
   m.def("stream_mix_norm", &stream_mix_norm);
   m.def("short_conv_residual", &short_conv_residual);

@@ -241,9 +241,11 @@ __global__ __launch_bounds__(256) void gelu_tanh_vec8_kernel(
 // and the pair only) are evaluated once into LDS, then the block's waves
 // walk the head slots — [0,H) query heads, [H,H+G) key heads, [H+G,H+2G)
 // value heads. q/k: RMS norm over the head (weight or none) then rotary on
-// the first 2*n_rot dims; v: turned by the row's position over all its dims
-// (n_vrot pairs; 0 = stored plain). Pairs are (2i,2i+1) when interleaved,
-// (i, i+n) otherwise. k and v go to their page.
+// the first 2*n_rot dims, cos and sin times rot_mag, then (norm_after) the
+// head divided by its root mean square once more, without a weight; v:
+// turned by the row's position over all its dims (n_vrot pairs; 0 = stored
+// plain). Pairs are (2i,2i+1) when interleaved, (i, i+n) otherwise. k and v
+// go to their page.
 constexpr int ROPE_MAX_PAIRS = 256;
 
 template <typename AT>
@@ -255,13 +257,17 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
     int n_rot, const float* __restrict__ freq_v, int n_vrot,
     AT* __restrict__ k_cache, AT* __restrict__ v_cache,
     const int64_t* __restrict__ slot_mapping, int H, int G, int D, int V,
-    int block_size, int interleaved) {
+    int block_size, int interleaved, float rot_mag, int norm_after) {
   __shared__ float cs_qk[ROPE_MAX_PAIRS][2];
   __shared__ float cs_v[ROPE_MAX_PAIRS][2];
   const int t = blockIdx.x;
   const float pos = (float)positions[t];
-  for (int i = threadIdx.x; i < n_rot; i += 256)
-    sincosf(pos * freq_qk[i], &cs_qk[i][1], &cs_qk[i][0]);
+  for (int i = threadIdx.x; i < n_rot; i += 256) {
+    float sn, cs;
+    sincosf(pos * freq_qk[i], &sn, &cs);
+    cs_qk[i][0] = cs * rot_mag;
+    cs_qk[i][1] = sn * rot_mag;
+  }
   for (int i = threadIdx.x; i < n_vrot; i += 256)
     sincosf(pos * freq_v[i], &cs_v[i][1], &cs_v[i][0]);
   __syncthreads();
@@ -293,6 +299,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
       }
     }
     const bool normed = nw != nullptr;
+    const bool after = norm_after && hs < H + G;
     // the head is read once: this lane's pairs stay in registers between
     // the sum of squares and the rotation (npairs <= 64 * 4)
     float pa[ROPE_MAX_PAIRS / 64], pb[ROPE_MAX_PAIRS / 64];
@@ -315,6 +322,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
       ss = wave_reduce_sum(ss);
       rstd = 1.f / sqrtf(ss / (float)n + eps);
     }
+    // the turned pairs replace the plain ones in the registers
+    float ss2 = 0.f;
 #pragma unroll
     for (int u = 0; u < ROPE_MAX_PAIRS / 64; ++u) {
       const int i = lane + 64 * u;
@@ -324,14 +333,35 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
         float a = pa[u] * rstd, b = pb[u] * rstd;
         if (normed) { a *= nw[d0]; b *= nw[d1]; }
         const float c = cs[i][0], sn = cs[i][1];
-        Act<AT>::st(dst + d0, a * c - b * sn);
-        Act<AT>::st(dst + d1, b * c + a * sn);
+        pa[u] = a * c - b * sn;
+        pb[u] = b * c + a * sn;
+        ss2 += pa[u] * pa[u] + pb[u] * pb[u];
+      }
+    }
+    float rstd2 = 1.f;
+    if (after) {
+      for (int i = 2 * npairs + lane; i < n; i += 64) {
+        float a = Act<AT>::ld(src + i) * rstd;
+        if (normed) a *= nw[i];
+        ss2 += a * a;
+      }
+      ss2 = wave_reduce_sum(ss2);
+      rstd2 = 1.f / sqrtf(ss2 / (float)n + eps);
+    }
+#pragma unroll
+    for (int u = 0; u < ROPE_MAX_PAIRS / 64; ++u) {
+      const int i = lane + 64 * u;
+      if (i < npairs) {
+        const int d0 = interleaved ? 2 * i : i;
+        const int d1 = interleaved ? 2 * i + 1 : i + npairs;
+        Act<AT>::st(dst + d0, pa[u] * rstd2);
+        Act<AT>::st(dst + d1, pb[u] * rstd2);
       }
     }
     for (int i = 2 * npairs + lane; i < n; i += 64) {
       float a = Act<AT>::ld(src + i) * rstd;
       if (normed) a *= nw[i];
-      Act<AT>::st(dst + i, a);
+      Act<AT>::st(dst + i, a * rstd2);
     }
   }
 }
@@ -449,7 +479,7 @@ extern "C" int arks_seq_qk_norm_rope_cache(
     const void* positions, const void* freq_qk, int n_rot, const void* freq_v,
     int n_vrot, void* k_cache, void* v_cache, const void* slot_mapping, int T,
     int H, int G, int D, int V, int block_size, int interleaved, int act_f32,
-    hipStream_t stream) {
+    float rot_mag, int norm_after, hipStream_t stream) {
   if (n_rot > ROPE_MAX_PAIRS || n_vrot > ROPE_MAX_PAIRS) return 1;
   if (T == 0) return 0;
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
@@ -458,6 +488,6 @@ extern "C" int arks_seq_qk_norm_rope_cache(
       (const float*)qw, (const float*)kw, eps, (const int64_t*)positions,
       (const float*)freq_qk, n_rot, (const float*)freq_v, n_vrot, (AT*)k_cache,
       (AT*)v_cache, (const int64_t*)slot_mapping, H, G, D, V, block_size,
-      interleaved));
+      interleaved, rot_mag, norm_after));
   return 0;
 }

@@ -2,11 +2,14 @@
 // feed-forward (arks_amd/models/feedforward.py GroupedMoE), bf16 or float
 // rows.
 //
-//   moe_route_grouped  softmax over all E experts in fp32; experts are cut into
+//   moe_route_grouped  scores over all E experts in fp32, their softmax or
+//       (sigmoid) each logit's own sigmoid; experts are cut into
 //       `groups` contiguous runs of E/groups, a run's score is its highest
 //       expert score and only the `keep` highest-scoring runs stay eligible; the `top`
-//       largest scores among those, divided by their sum (+1e-20). Ties go
-//       to the lower index (groups and experts).
+//       largest scores among those, divided by their sum (+1e-20) unless
+//       renorm is off. Ties go to the lower index (groups and experts).
+//       matrix (optional, [T, E]): the row's weights at the experts it uses,
+//       0 elsewhere.
 //   moe_mix_rows  out[t] = sum_j w[t][j] * y[row(t, j)], row given, or
 //       ids[t][j] * T + t for dense per-expert outputs y [E, T, H].
 #include "seq_common.h"
@@ -21,24 +24,31 @@ constexpr int ROUTE_MAX_K = 32;
 // One wave per row.
 __global__ __launch_bounds__(64) void moe_route_grouped_kernel(
     float* __restrict__ weights, int* __restrict__ ids,
-    const float* __restrict__ logits, int E, int top, int groups, int keep) {
+    const float* __restrict__ logits, int E, int top, int groups, int keep,
+    int sigmoid, int renorm, float* __restrict__ matrix) {
   __shared__ float s_s[ROUTE_MAX_E];
   __shared__ float g_s[ROUTE_MAX_E];  // group scores (groups <= E)
   const int t = blockIdx.x, lane = threadIdx.x;
   const float* row = logits + (int64_t)t * E;
-  float m = -FLT_MAX;
-  for (int e = lane; e < E; e += 64) m = fmaxf(m, row[e]);
-  m = wave_reduce_max(m);
-  float sum = 0.f;
-  for (int e = lane; e < E; e += 64) {
-    const float p = expf(row[e] - m);
-    s_s[e] = p;
-    sum += p;
+  if (sigmoid) {
+    for (int e = lane; e < E; e += 64) s_s[e] = sigmoid_f(row[e]);
+  } else {
+    float m = -FLT_MAX;
+    for (int e = lane; e < E; e += 64) m = fmaxf(m, row[e]);
+    m = wave_reduce_max(m);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) {
+      const float p = expf(row[e] - m);
+      s_s[e] = p;
+      sum += p;
+    }
+    sum = wave_reduce_sum(sum);
+    __syncthreads();
+    const float inv = 1.f / sum;
+    for (int e = lane; e < E; e += 64) s_s[e] *= inv;
   }
-  sum = wave_reduce_sum(sum);
-  __syncthreads();
-  const float inv = 1.f / sum;
-  for (int e = lane; e < E; e += 64) s_s[e] *= inv;
+  if (matrix)
+    for (int e = lane; e < E; e += 64) matrix[(int64_t)t * E + e] = 0.f;
   __syncthreads();
   const int per = E / groups;
   for (int gI = lane; gI < groups; gI += 64) {
@@ -97,8 +107,10 @@ __global__ __launch_bounds__(64) void moe_route_grouped_kernel(
   if (lane == 0) {
     const float d = wsum + 1e-20f;
     for (int r = 0; r < top; ++r) {
-      weights[(int64_t)t * top + r] = wk[r] / d;
+      const float w = renorm ? wk[r] / d : wk[r];
+      weights[(int64_t)t * top + r] = w;
       ids[(int64_t)t * top + r] = ik[r];
+      if (matrix) matrix[(int64_t)t * E + ik[r]] = w;
     }
   }
 }
@@ -107,10 +119,10 @@ template <typename AT>
 __global__ __launch_bounds__(256) void moe_mix_rows_kernel(
     AT* __restrict__ out, const AT* __restrict__ y,
     const float* __restrict__ weights, const int* __restrict__ rows, int T,
-    int H, int k, int dense) {
+    int H, int k, int dense, const AT* __restrict__ add) {
   const int t = blockIdx.x;
   for (int c = threadIdx.x; c < H; c += 256) {
-    float acc = 0.f;
+    float acc = add ? Act<AT>::ld(add + (int64_t)t * H + c) : 0.f;
     for (int j = 0; j < k; ++j) {
       const int64_t r = dense ? (int64_t)rows[t * k + j] * T + t
                               : (int64_t)rows[t * k + j];
@@ -124,12 +136,18 @@ __global__ __launch_bounds__(256) void moe_mix_rows_kernel(
 __global__ __launch_bounds__(256) void moe_mix_rows_vec8_kernel(
     bf16* __restrict__ out, const bf16* __restrict__ y,
     const float* __restrict__ weights, const int* __restrict__ rows, int T,
-    int H, int k, int dense) {
+    int H, int k, int dense, const bf16* __restrict__ add) {
   const int t = blockIdx.x;
   for (int c = threadIdx.x * 8; c < H; c += 256 * 8) {
     float acc[8];
+    if (add) {
+      const ushort8 u = *reinterpret_cast<const ushort8*>(add + (int64_t)t * H + c);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+      for (int e = 0; e < 8; ++e) acc[e] = bf16_bits_to_float(u[e]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    }
     for (int j = 0; j < k; ++j) {
       const int64_t r = dense ? (int64_t)rows[t * k + j] * T + t
                               : (int64_t)rows[t * k + j];
@@ -152,29 +170,32 @@ using namespace arks;
 extern "C" int arks_seq_moe_route_grouped(void* weights, void* ids,
                                           const void* logits, int T, int E,
                                           int top, int groups, int keep,
-                                          hipStream_t stream) {
+                                          int sigmoid, int renorm,
+                                          void* matrix, hipStream_t stream) {
   if (E > ROUTE_MAX_E || top > ROUTE_MAX_K || groups < 1 || E % groups ||
       keep > groups || top > keep * (E / groups))
     return 1;
   if (T == 0) return 0;
   hipLaunchKernelGGL(moe_route_grouped_kernel, dim3(T), dim3(64), 0, stream,
                      (float*)weights, (int*)ids, (const float*)logits, E, top,
-                     groups, keep);
+                     groups, keep, sigmoid, renorm, (float*)matrix);
   return 0;
 }
 
 extern "C" void arks_seq_moe_mix_rows(void* out, const void* y,
                                       const void* weights, const void* rows,
                                       int T, int H, int k, int dense,
-                                      int act_f32, hipStream_t stream) {
+                                      const void* add, int act_f32,
+                                      hipStream_t stream) {
   if (T == 0) return;
   if (!act_f32 && H % 8 == 0) {
     hipLaunchKernelGGL(moe_mix_rows_vec8_kernel, dim3(T), dim3(256), 0, stream,
                        (bf16*)out, (const bf16*)y, (const float*)weights,
-                       (const int*)rows, T, H, k, dense);
+                       (const int*)rows, T, H, k, dense, (const bf16*)add);
     return;
   }
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
       (moe_mix_rows_kernel<AT>), dim3(T), dim3(256), 0, stream, (AT*)out,
-      (const AT*)y, (const float*)weights, (const int*)rows, T, H, k, dense));
+      (const AT*)y, (const float*)weights, (const int*)rows, T, H, k, dense,
+      (const AT*)add));
 }

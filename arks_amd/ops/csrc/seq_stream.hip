@@ -369,32 +369,36 @@ __device__ __forceinline__ float glu_value(float g, float u, int mode,
 template <typename AT>
 __global__ __launch_bounds__(256) void glu_act_kernel(
     AT* __restrict__ out, int64_t ldo, const AT* __restrict__ gu, int64_t ldg,
-    int64_t rows, int F, int mode, float limit, float alpha) {
+    int64_t rows, int F, int mode, float limit, float alpha,
+    const float* __restrict__ row_scale) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= rows * F) return;
   const int64_t t = i / F;
   const int c = (int)(i - t * F);
-  const float g = Act<AT>::ld(gu + t * ldg + c);
-  const float u = Act<AT>::ld(gu + t * ldg + F + c);
+  const float rs = row_scale ? row_scale[t] : 1.f;
+  const float g = rs * Act<AT>::ld(gu + t * ldg + c);
+  const float u = rs * Act<AT>::ld(gu + t * ldg + F + c);
   Act<AT>::st(out + t * ldo + c, glu_value(g, u, mode, limit, alpha));
 }
 
 // bf16, 8 elements per thread (F % 8 == 0, 16-byte aligned rows)
 __global__ __launch_bounds__(256) void glu_act_vec8_kernel(
     bf16* __restrict__ out, int64_t ldo, const bf16* __restrict__ gu,
-    int64_t ldg, int64_t rows, int F, int mode, float limit, float alpha) {
+    int64_t ldg, int64_t rows, int F, int mode, float limit, float alpha,
+    const float* __restrict__ row_scale) {
   const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
   if (i >= rows * F) return;
   const int64_t t = i / F;
   const int c = (int)(i - t * F);
+  const float rs = row_scale ? row_scale[t] : 1.f;
   const ushort8 gv = *reinterpret_cast<const ushort8*>(gu + t * ldg + c);
   const ushort8 uv = *reinterpret_cast<const ushort8*>(gu + t * ldg + F + c);
   ushort8 o;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    o[e] = float_to_bf16_bits(glu_value(bf16_bits_to_float(gv[e]),
-                                        bf16_bits_to_float(uv[e]), mode, limit,
-                                        alpha));
+    o[e] = float_to_bf16_bits(glu_value(rs * bf16_bits_to_float(gv[e]),
+                                        rs * bf16_bits_to_float(uv[e]), mode,
+                                        limit, alpha));
   }
   *reinterpret_cast<ushort8*>(out + t * ldo + c) = o;
 }
@@ -490,7 +494,8 @@ extern "C" void arks_seq_head_norm_gate(void* out, int64_t ldo, const void* o,
 
 extern "C" void arks_seq_glu_act(void* out, int64_t ldo, const void* gu,
                                  int64_t ldg, int64_t rows, int F, int mode,
-                                 float limit, float alpha, int act_f32,
+                                 float limit, float alpha,
+                                 const void* row_scale, int act_f32,
                                  hipStream_t stream) {
   const int64_t n = rows * F;
   if (n == 0) return;
@@ -499,10 +504,11 @@ extern "C" void arks_seq_glu_act(void* out, int64_t ldo, const void* gu,
     hipLaunchKernelGGL(glu_act_vec8_kernel,
                        dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0,
                        stream, (bf16*)out, ldo, (const bf16*)gu, ldg, rows, F,
-                       mode, limit, alpha);
+                       mode, limit, alpha, (const float*)row_scale);
     return;
   }
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
       (glu_act_kernel<AT>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
-      stream, (AT*)out, ldo, (const AT*)gu, ldg, rows, F, mode, limit, alpha));
+      stream, (AT*)out, ldo, (const AT*)gu, ldg, rows, F, mode, limit, alpha,
+      (const float*)row_scale));
 }
