@@ -123,6 +123,8 @@ def main(argv=None) -> int:
             print(e, file=sys.stderr)
             return 3
         raise
+    print(f"trace_run: {engine.model_cfg.architecture} in {a.dtype} on "
+          f"{engine.runner.device}", file=sys.stderr, flush=True)
     replay(engine, sys.stdin, a.out, log=proto)
     return 0
 

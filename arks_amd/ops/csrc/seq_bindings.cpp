@@ -158,7 +158,8 @@ int arks_seq_attn_masked_mfma(void* out, int64_t ldo, const void* q,
                               int window, int keep_first, float out_scale,
                               int T, int H, int G, int D, int V, int bs,
                               int max_blocks, int num_seqs, int single_rows,
-                              void* ws, int ksplit, hipStream_t stream);
+                              void* ws, int ksplit, int maps,
+                              hipStream_t stream);
 int arks_seq_attn_masked_ksplit(int T, int H, int G, int max_blocks);
 int arks_seq_moe_route_grouped(void* weights, void* ids, const void* logits,
                                int T, int E, int top, int groups, int keep,
@@ -1297,16 +1298,20 @@ bool attention_masked_mfma(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
                            Tensor token_seq, double scale, OptTensor sink_w,
                            double softcap, int64_t window, int64_t keep_first,
                            double out_scale, bool single_rows, int64_t maps) {
-  if (maps != 1) return false;
   TORCH_CHECK(q.is_cuda() && q.scalar_type() == torch::kBFloat16 &&
-              q.is_contiguous() && q.dim() == 3);
+              q.is_contiguous() && q.dim() == 3 && maps >= 1);
   const int T = q.size(0), H = q.size(1), D = q.size(2);
   TORCH_CHECK(k_cache.scalar_type() == q.scalar_type() &&
               v_cache.scalar_type() == q.scalar_type() &&
               out.scalar_type() == q.scalar_type());
-  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(3) == D);
-  const int G = k_cache.size(1), bs = k_cache.size(2), V = v_cache.size(3);
-  TORCH_CHECK(H % G == 0 && v_cache.size(1) == G && v_cache.size(2) == bs);
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 &&
+              k_cache.size(3) == D * maps);
+  // key groups: every key/value head of the cache once per map
+  const int G = k_cache.size(1) * maps, bs = k_cache.size(2),
+            V = v_cache.size(3);
+  TORCH_CHECK(H % G == 0 && v_cache.size(1) * maps == G &&
+              v_cache.size(2) == bs);
+  TORCH_CHECK(maps == 1 || !sink_w.has_value());
   const int64_t ldk = paged_row_stride(k_cache, "k_cache");
   const int64_t ldv = paged_row_stride(v_cache, "v_cache");
   const int64_t ldo = head_row_stride(out, "out");
@@ -1337,7 +1342,7 @@ bool attention_masked_mfma(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
              (float)scale, sw_p, (float)softcap, (int)window, (int)keep_first,
              (float)out_scale, T, H, G, D, V, bs, (int)block_tables.size(1),
              m.S, single_rows ? 1 : 0, ksplit > 1 ? ws.data_ptr() : nullptr,
-             ksplit, current_stream()) == 0;
+             ksplit, (int)maps, current_stream()) == 0;
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {

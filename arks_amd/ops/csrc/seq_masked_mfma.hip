@@ -21,7 +21,9 @@
 //     start from a sink (max sink[h], sum 1);
 //   * key and value rows have strides of their own (ldk, ldv);
 //   * no host work list: a workgroup finds its (sequence, first position)
-//     by walking cu_seqlens, or — steps of single rows — from token_seq.
+//     by walking cu_seqlens, or — steps of single rows — from token_seq;
+//   * a cache row may hold several keys side by side that share its value
+//     (MaskArgs::maps): each is a key group of its own with its own heads.
 #include "seq_common.h"
 
 #include <cfloat>
@@ -46,6 +48,10 @@ __device__ __forceinline__ float mk_cap(float s, float cap, float inv_cap) {
 struct MaskArgs {
   float scale, softcap, out_scale;
   int window, keep_first;  // window: INT_MAX / 2 when there is none
+  // key maps per cache row: a row holds `maps` keys of D dims side by side
+  // that share the row's value; the kernels' G counts (key/value head, map)
+  // groups, group g reads key g % maps of the rows of head g / maps
+  int maps;
 };
 
 template <int D, int V>  // V: the value columns one workgroup holds
@@ -110,6 +116,8 @@ void attn_masked_tile_kernel(
   const int hblocks = GQ >> hpt_shift;  // head blocks per key/value head
   const int kvh = (blockIdx.x / VS) / hblocks;
   const int h0 = kvh * GQ + ((blockIdx.x / VS) % hblocks) * HPT;
+  const int GR = G / a.maps, kvr = kvh / a.maps;  // heads of rows, this one
+  const bf16* __restrict__ k_rows = k_cache + (kvh % a.maps) * D;
   const int q_start = cu[seq_idx];
   const int q_len = cu[seq_idx + 1] - q_start;
   const int kv_len = kv_lens[seq_idx];
@@ -179,9 +187,9 @@ void attn_masked_tile_kernel(
       ushort8 kv{};
       if (i < MK_KTILE * (D / 8) && kg < kmax) {
         const int64_t row =
-            ((int64_t)(key < MK_PAGE ? pg0 : pg1) * G + kvh) * MK_PAGE +
+            ((int64_t)(key < MK_PAGE ? pg0 : pg1) * GR + kvr) * MK_PAGE +
             kg % MK_PAGE;
-        kv = *reinterpret_cast<const ushort8*>(k_cache + row * ldk + col8);
+        kv = *reinterpret_cast<const ushort8*>(k_rows + row * ldk + col8);
       }
       kld[j] = kv;
     }
@@ -195,7 +203,7 @@ void attn_masked_tile_kernel(
         ushort8 vv{};
         if (i < MK_KTILE * (V / 8) && kg < kmax) {
           const int64_t row =
-              ((int64_t)(key < MK_PAGE ? pg0 : pg1) * G + kvh) * MK_PAGE +
+              ((int64_t)(key < MK_PAGE ? pg0 : pg1) * GR + kvr) * MK_PAGE +
               kg % MK_PAGE;
           vv = *reinterpret_cast<const ushort8*>(v_cache + row * ldv + voff +
                                                  col8);
@@ -420,6 +428,8 @@ __global__ __launch_bounds__(256, 2) void attn_masked_dec_kernel(
   constexpr int E = V / 16;  // value dims per thread in the merge
   const int t = blockIdx.y, kvh = blockIdx.x;
   const int GQ = H / G;
+  const int GR = G / a.maps, kvr = kvh / a.maps;
+  const bf16* __restrict__ k_rows = k_cache + (kvh % a.maps) * D;
   const int seq = token_seq[t];
   const int q_start = cu[seq];
   const int pos = kv_lens[seq] - (cu[seq + 1] - q_start) + (t - q_start);
@@ -482,7 +492,7 @@ __global__ __launch_bounds__(256, 2) void attn_masked_dec_kernel(
                        ushort8 (&vr)[NV]) {
     const int key_base = tile_base(it);
     auto row_of = [&](int key) -> int64_t {  // key within the tile
-      return ((int64_t)(key < MK_PAGE ? p0 : p1) * G + kvh) * MK_PAGE +
+      return ((int64_t)(key < MK_PAGE ? p0 : p1) * GR + kvr) * MK_PAGE +
              key % MK_PAGE;
     };
 #pragma unroll
@@ -500,7 +510,7 @@ __global__ __launch_bounds__(256, 2) void attn_masked_dec_kernel(
     for (int sub = 0; sub < 2; ++sub) {
       const int key = sub * 16 + lq;
       const bool have = key_base + key < kmax;
-      const bf16* krow = k_cache + (have ? row_of(key) : 0) * ldk + 8 * la;
+      const bf16* krow = k_rows + (have ? row_of(key) : 0) * ldk + 8 * la;
 #pragma unroll
       for (int st = 0; st < STEPS; ++st) {
         ushort8 u{};
@@ -723,7 +733,10 @@ extern "C" int arks_seq_attn_masked_mfma(
     const void* seq_lens, const void* cu, const void* token_seq, float scale,
     const void* sink_w, float softcap, int window, int keep_first,
     float out_scale, int T, int H, int G, int D, int V, int bs, int max_blocks,
-    int num_seqs, int single_rows, void* ws, int ksplit, hipStream_t stream) {
+    int num_seqs, int single_rows, void* ws, int ksplit, int maps,
+    hipStream_t stream) {
+  // G: key groups, maps of them per key/value head of the cache
+  if (maps < 1 || G % maps || (maps > 1 && v_cache == k_cache)) return 1;
   if (bs != MK_PAGE || H % G || ldk % 8 || ldv % 8 || ldo % 8 ||
       ((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) ||
       ((uintptr_t)v_cache & 15) || ((uintptr_t)out & 15))
@@ -736,6 +749,7 @@ extern "C" int arks_seq_attn_masked_mfma(
   a.out_scale = out_scale;
   a.window = window > 0 ? window : (1 << 30);
   a.keep_first = window > 0 ? keep_first : 0;
+  a.maps = maps;
   const bool shared_rows = v_cache == k_cache && ldv == ldk;
   const int hpt_shift = masked_hpt_shift(GQ);
   const int ppt = MK_QTILE >> hpt_shift;

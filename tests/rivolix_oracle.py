@@ -165,12 +165,16 @@ def expert(h, w):
     return (silu(h @ w["gate"].T) * (h @ w["up"].T)) @ w["down"].T
 
 
-def routed_experts(h, w, mlp):
+def routed_experts(h, w, mlp, margins=None):
     """Scores sigmoid(W_router h); the `top` highest-scoring experts run on
     score * h and their results are summed as they are; the shared expert
-    runs on h."""
+    runs on h. margins (a list) receives, per row, how far the last chosen
+    score lies above the first one left out."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
     s = sigmoid(h @ w["router"].T)
+    if margins is not None and E > top:
+        ranked = torch.sort(s, -1, descending=True).values
+        margins.append(ranked[:, top - 1] - ranked[:, top])
     out = torch.zeros(h.shape[0], w["e0.down"].shape[0], dtype=F64)
     chosen = torch.topk(s, top, dim=-1).indices
     for t in range(h.shape[0]):
@@ -186,7 +190,7 @@ def sub(weights, prefix):
     return {k[len(prefix):]: v for k, v in weights.items() if k.startswith(prefix)}
 
 
-def forward(cfg, weights, tokens):
+def forward(cfg, weights, tokens, margins=None):
     eps = cfg["norm"]["eps"]
     x = weights["embed"][torch.tensor(tokens)].clone()
     after, kept = [], {}
@@ -206,11 +210,29 @@ def forward(cfg, weights, tokens):
         y = y * lw["ls1"]
         if spec.get("mlp") is not None:
             h2 = offset_norm(x, lw["norm2"], eps)
-            y = y + routed_experts(h2, sub(lw, "mlp."), spec["mlp"]) * lw["ls2"]
+            y = y + routed_experts(h2, sub(lw, "mlp."), spec["mlp"],
+                                   margins) * lw["ls2"]
         x = x + y
         after.append(x.clone())
     xn = offset_norm(x, weights["final.norm"], eps)
     return xn @ weights["embed"].T, after
+
+
+def clear_choices(cfg, weights, tokens, least=0.008, after=3):
+    """Rows at which, and for `after` rows before which, every layer's
+    router chooses by a margin of at least `least`: a run in reduced
+    precision may choose otherwise at a close call, and then computes
+    another function at that row and, through the convolutions' taps and the
+    newest keys, near it."""
+    margins = []
+    forward(cfg, weights, tokens, margins)
+    ok = torch.ones(len(tokens), dtype=torch.bool)
+    for m in margins:
+        ok &= m >= least
+    near = ok.clone()
+    for d in range(1, after + 1):
+        near[d:] &= ok[:-d]
+    return near
 
 
 # ------------------------------------------------------- configs and weights

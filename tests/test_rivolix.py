@@ -1,0 +1,724 @@
+"""Rivolix through the engine, and its mechanisms one by one, against the
+plain float64 model of tests/rivolix_oracle.py.
+
+Engine cases write a small random checkpoint, build an engine on it and
+replay a step plan with the product's trace replay (the scheduler's pages
+and state slots, the runner's batches, the model's kernels); op cases drive
+single ops with inputs made so that a fault shows (one key that must win in
+one of the two maps only, far back and on both sides of a page border; a
+difference weight that cancels a map; convolution histories over one- and
+two-row portions into junk-filled slots; query factors on both sides of a
+step of the logarithm; an expert whose score scales its input). CPU cases
+run the reference ops, gpu-marked ones the HIP kernels in float32 and
+bfloat16.
+"""
+
+import io
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import rivolix_oracle as O
+
+CASES = [
+    pytest.param("cpu", "float32", id="cpu-f32"),
+    pytest.param("cuda", "float32", id="gpu-f32", marks=pytest.mark.gpu),
+    pytest.param("cuda", "bfloat16", id="gpu-bf16", marks=pytest.mark.gpu),
+]
+GPU_CASES = [c for c in CASES if c.id != "cpu-f32"]
+TOL = {"float32": 2e-4, "bfloat16": 6e-2}
+TDT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+F64 = torch.float64
+
+D, K, MOE = O.difference_spec, O.key_value_spec, O.moe_spec
+
+
+# ------------------------------------------------------------------ helpers
+def write_checkpoint(path, cfg, seed=0):
+    from safetensors.torch import save_file
+
+    os.makedirs(path, exist_ok=True)
+    w = O.random_weights(cfg, seed)
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in w.items()},
+              os.path.join(path, "model.safetensors"))
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    return w
+
+
+def make_engine(path, device, dtype, max_tokens=256, **kw):
+    from arks_amd.config import EngineConfig
+    from arks_amd.engine import LLMEngine
+
+    cfg = EngineConfig(model_path=str(path), device=device, dtype=dtype,
+                       kv_cache_blocks=-(-max_tokens // 16), max_num_seqs=4,
+                       max_model_len=max_tokens, max_num_batched_tokens=max_tokens,
+                       enable_prefix_caching=False, **kw)
+    return LLMEngine(cfg)
+
+
+def replay(engine, tmp_path, steps):
+    """steps: lists of (request id, tokens, end?); logits of every token.
+    Returns {id: [n_tokens, vocab]}."""
+    from arks_amd.engine.trace import replay as trace_replay
+
+    out = tmp_path / "out"
+    out.mkdir(exist_ok=True)
+    lines = [json.dumps({
+        "step": n,
+        "entries": [{"id": i, "tokens": t, "want": list(range(len(t)))}
+                    for i, t, _ in step],
+        "end": [i for i, _, e in step if e]}) for n, step in enumerate(steps)]
+    trace_replay(engine, lines, str(out), log=io.StringIO())
+    got = {}
+    V = engine.model_cfg.vocab_size
+    for n, step in enumerate(steps):
+        arr = np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, V)
+        at = 0
+        for i, t, _ in step:
+            got.setdefault(i, []).append(arr[at:at + len(t)])
+            at += len(t)
+    return {i: np.concatenate(v) for i, v in got.items()}
+
+
+def rel_err(got, want):
+    """Largest row error over the rms of all logits."""
+    want = want.numpy() if isinstance(want, torch.Tensor) else want
+    d = got - want
+    return float((np.sqrt((d ** 2).mean(-1)) / np.sqrt((want ** 2).mean())).max())
+
+
+def portions(tokens, sizes):
+    out, at, k = [], 0, 0
+    while at < len(tokens):
+        n = sizes[k % len(sizes)]
+        out.append(tokens[at:at + n])
+        at += n
+        k += 1
+    return out
+
+
+def toks(n, vocab=96, seed=1):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def oracle_logits(cfg, w, t):
+    return O.forward(cfg, w, t)[0]
+
+
+def assert_logits(got, cfg, w, t, dtype, note=None):
+    """got [n, vocab] against the oracle's first n rows. bfloat16 runs are
+    compared at the rows where no router's choice is a close call (the
+    oracle says which, with the rows just behind one): a flipped choice is
+    another function, not an error of rounding."""
+    n = got.shape[0]
+    want = oracle_logits(cfg, w, t)[:n]
+    if dtype == "bfloat16":
+        # whatever is left out, the typical row must be well inside
+        rows = np.sqrt(((got - want.numpy()) ** 2).mean(-1))
+        assert np.median(rows) / float(want.pow(2).mean().sqrt()) < TOL[dtype] / 3, note
+        keep = O.clear_choices(cfg, w, t)[:n].numpy()
+        if not keep.any():
+            return
+        got, want = got[keep], want[torch.from_numpy(keep)]
+    assert rel_err(got, want) < TOL[dtype], note
+
+
+# --------------------------------------------------- the model in the engine
+ONE_LAYER = {
+    "difference": [D()],
+    "difference-alone": [D(mlp=None)],
+    "key-valued": [K()],
+    "key-valued-alone": [K(mlp=None)],
+    "borrowed-keys": [D(), D(kv_from=0)],
+    "borrowed-keys-alone": [D(mlp=None), D(kv_from=0, mlp=None)],
+}
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("name", list(ONE_LAYER))
+def test_one_mixer(tmp_path, device, dtype, name):
+    cfg = O.make_config(ONE_LAYER[name])
+    w = write_checkpoint(tmp_path / "m", cfg)
+    t = toks(45)
+    eng = make_engine(tmp_path / "m", device, dtype)
+    got = replay(eng, tmp_path, [[("a", t, True)]])["a"]
+    assert_logits(got, cfg, w, t, dtype)
+
+
+def model_config():
+    """Both mixers, a layer on borrowed keys behind a layer of another kind
+    (the pages it reads are two layers back), query factors that step every
+    five positions, four taps of history crossed by short portions."""
+    return O.make_config([D(), K(), D(kv_from=0), D(conv=2, every=7, mlp=None),
+                          K(rot_dims=16, scaling=None, mlp=MOE(top=1))])
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_residual_after_every_layer(tmp_path, device, dtype):
+    cfg = model_config()
+    w = write_checkpoint(tmp_path / "m", cfg)
+    t = toks(23)
+    _, after = O.forward(cfg, w, t)
+    eng = make_engine(tmp_path / "m", device, dtype)
+    seen = {}
+    eng.runner.model.residual_tap = lambda i, x: seen.__setitem__(
+        i, x.detach().clone().float().cpu())
+    replay(eng, tmp_path, [[("a", t, True)]])
+    assert sorted(seen) == list(range(len(after)))
+    for i, want in enumerate(after):
+        err = (seen[i].double() - want).abs().max() / want.abs().max()
+        assert float(err) < (1e-4 if dtype == "float32" else 4e-2), i
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_prefill_against_decode_and_portions(tmp_path, device, dtype):
+    cfg = model_config()
+    w = write_checkpoint(tmp_path / "m", cfg)
+    t = toks(70)
+    for name, plan in {
+        "decode": [t[:9]] + [[x] for x in t[9:]],
+        "small": portions(t, [2, 3, 5, 2, 7]),
+        "pairs": portions(t, [2]),
+        "odd": portions(t, [13, 1, 2, 17]),
+        "tokens": [[x] for x in t[:40]],
+    }.items():
+        eng = make_engine(tmp_path / "m", device, dtype)
+        steps = [[("a", p, False)] for p in plan]
+        got = replay(eng, tmp_path, steps)["a"]
+        assert_logits(got, cfg, w, t, dtype, name)
+
+
+def mixed_plan(reqs, slots, pool_pages, sizes):
+    """Steps in which unequal requests run side by side, portions beside
+    single tokens, some sitting a step out; never more than `slots` live
+    and never more pages than the pool holds."""
+    at = {c: 0 for c in reqs}
+    live, waiting, steps = [], list(reqs), []
+    k = 0
+    while live or waiting:
+        while waiting and len(live) < slots and \
+                sum(-(-len(reqs[c]) // 16) for c in live + waiting[:1]) <= pool_pages:
+            live.append(waiting.pop(0))
+        step = []
+        for c in list(live):
+            if (k + ord(c)) % 5 == 0 and len(live) > 1:
+                k += 1
+                continue  # this request sits the step out
+            n = min(sizes[k % len(sizes)], len(reqs[c]) - at[c])
+            k += 1
+            part = reqs[c][at[c]:at[c] + n]
+            at[c] += n
+            done = at[c] == len(reqs[c])
+            step.append((c, part, done))
+            if done:
+                live.remove(c)
+        if step:
+            steps.append(step)
+    return steps
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_mixed_batches_and_reuse(tmp_path, device, dtype):
+    """More requests than state slots over time and a pool just large
+    enough, so pages and slots are given back and taken again."""
+    cfg = model_config()
+    w = write_checkpoint(tmp_path / "m", cfg)
+    reqs = {c: toks(n, seed=s) for c, n, s in
+            [("a", 61, 1), ("b", 18, 2), ("c", 33, 3), ("d", 5, 4),
+             ("e", 47, 5), ("f", 29, 6), ("g", 40, 7)]}
+    steps = mixed_plan(reqs, 4, 12, [7, 1, 2, 16, 1, 1, 3, 11])
+    eng = make_engine(tmp_path / "m", device, dtype, max_tokens=192)
+    got = replay(eng, tmp_path, steps)
+    for c in reqs:
+        assert got[c].shape[0] == len(reqs[c])
+        assert_logits(got[c], cfg, w, reqs[c], dtype, c)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_long_decode(tmp_path, device, dtype):
+    """150 single tokens: the query factor passes 30 steps of its
+    logarithm, ten pages fill up one token at a time."""
+    cfg = O.make_config([D(), K(), D(kv_from=0, mlp=None)])
+    w = write_checkpoint(tmp_path / "m", cfg)
+    t = toks(150)
+    eng = make_engine(tmp_path / "m", device, dtype)
+    steps = [[("a", t[:5], False)]] + [[("a", [x], False)] for x in t[5:]]
+    got = replay(eng, tmp_path, steps)["a"]
+    assert_logits(got, cfg, w, t, dtype)
+
+
+OTHER_SIZES = {
+    "one-kv-head": dict(layers=[D(heads=6, kv_heads=1, dim=8, vdim=12)]),
+    "all-kv-heads": dict(layers=[D(heads=3, kv_heads=3, dim=12, vdim=4),
+                                 K(heads=3, kv_heads=3, dim=8, rot_dims=8)]),
+    "no-history": dict(layers=[D(conv=1), D(conv=1, kv_from=0)]),
+    "eight-taps": dict(layers=[D(conv=8), D(conv=8, kv_from=0)]),
+    "no-difference": dict(layers=[D(diff=0.0)]),
+    "large-difference": dict(layers=[D(diff=0.8)]),
+    "factor-every-position": dict(layers=[D(every=1, coef=0.9)]),
+    "factor-never": dict(layers=[D(every=100000)]),
+    "factor-off": dict(layers=[D(coef=0.0)]),
+    "wide-values": dict(layers=[D(heads=2, kv_heads=1, dim=4, vdim=72)]),
+    "sharp-scores": dict(layers=[D(scale=2.5), K(scale=9.0)]),
+    "two-borrowers": dict(layers=[D(), D(kv_from=0), K(), D(kv_from=0)]),
+    "borrow-from-later-owner": dict(layers=[D(), D(dim=16, vdim=8),
+                                            D(dim=16, vdim=8, kv_from=1)]),
+    "rotary-all-dims": dict(layers=[K(dim=8, rot_dims=8)]),
+    "rotary-two-dims": dict(layers=[K(rot_dims=2, base=7.0)]),
+    "rotary-none": dict(layers=[K(rot_dims=0)]),
+    "rotary-unscaled": dict(layers=[K(scaling=None)]),
+    "rotary-all-scaled": dict(layers=[K(scaling={
+        "factor": 16.0, "original": 4, "fast": 64.0, "slow": 32.0})]),
+    "rotary-ramp-inside": dict(layers=[K(dim=32, rot_dims=32, base=100.0, scaling={
+        "factor": 3.0, "original": 64, "fast": 6.0, "slow": 0.5})]),
+    "top-one": dict(layers=[D(mlp=MOE(top=1))]),
+    "top-all": dict(layers=[K(mlp=MOE(experts=3, top=3))]),
+    "one-expert": dict(layers=[K(mlp=MOE(experts=1, top=1))]),
+    "no-shared-expert": dict(layers=[D(mlp=MOE(shared_ff=0))]),
+    "many-experts": dict(layers=[K(mlp=MOE(experts=70, top=5, ff=8,
+                                           shared_ff=8))]),
+    "odd-everything": dict(layers=[
+        D(heads=3, kv_heads=1, dim=6, vdim=10, conv=3, every=3,
+          mlp=MOE(experts=5, top=2, ff=14, shared_ff=22)),
+        K(heads=5, kv_heads=1, dim=10, rot_dims=6,
+          mlp=MOE(experts=7, top=3, ff=9, shared_ff=3)),
+        D(heads=3, kv_heads=1, dim=6, vdim=10, conv=3, kv_from=0, mlp=None)],
+        width=44, vocab=97, eps=1e-3),
+}
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("name", list(OTHER_SIZES))
+def test_other_sizes(tmp_path, device, dtype, name):
+    cfg = O.make_config(**OTHER_SIZES[name])
+    w = write_checkpoint(tmp_path / "m", cfg, seed=3)
+    t = toks(38, vocab=cfg["vocab"], seed=9)
+    eng = make_engine(tmp_path / "m", device, dtype)
+    steps = [[("a", p, False)] for p in portions(t, [11, 2, 1, 6])]
+    got = replay(eng, tmp_path, steps)["a"]
+    assert_logits(got, cfg, w, t, dtype)
+
+
+def fast_path_config():
+    """Sizes the vectorised and matrix-core kernels are built for."""
+    return O.make_config(
+        [D(heads=4, kv_heads=2, dim=64, vdim=64, conv=4, every=50),
+         K(heads=4, kv_heads=2, dim=64, rot_dims=32,
+           mlp=MOE(experts=8, top=2, ff=32, shared_ff=64)),
+         D(heads=4, kv_heads=2, dim=64, vdim=64, conv=4, every=50, kv_from=0),
+         D(heads=2, kv_heads=1, dim=128, vdim=128, conv=3, mlp=None),
+         K(heads=2, kv_heads=1, dim=128, rot_dims=128, mlp=None)],
+        width=64)
+
+
+@pytest.mark.parametrize("device,dtype", GPU_CASES)
+def test_fast_path_sizes(tmp_path, device, dtype):
+    """Prompts across 64-row tile edges, single rows after them, a step
+    above the row count at which the experts run sorted segments."""
+    cfg = fast_path_config()
+    w = write_checkpoint(tmp_path / "m", cfg)
+    t = toks(330, seed=11)
+    eng = make_engine(tmp_path / "m", device, dtype, max_tokens=512)
+    plan = [t[:130], t[130:131], t[131:197], t[197:198], t[198:199],
+            t[199:201], t[201:]]
+    assert len(plan[-1]) > 120
+    got = replay(eng, tmp_path, [[("a", p, False)] for p in plan])["a"]
+    assert_logits(got, cfg, w, t, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_sorted_expert_segments(tmp_path, device, dtype, monkeypatch):
+    """Steps above DENSE_TOKENS rows sort (row, expert) pairs by expert;
+    below they run every expert with factor 0 where unused: same logits."""
+    from arks_amd.models.feedforward import InputScaledMoE
+
+    monkeypatch.setattr(InputScaledMoE, "DENSE_TOKENS", 6)
+    cfg = O.make_config([D(mlp=MOE(experts=5, top=3)),
+                         K(mlp=MOE(experts=4, top=1, shared_ff=0))])
+    w = write_checkpoint(tmp_path / "m", cfg)
+    ta, tb = toks(50, seed=2), toks(31, seed=3)
+    eng = make_engine(tmp_path / "m", device, dtype)
+    steps = [[("a", ta[:21], False)], [("a", ta[21:24], False), ("b", tb[:30], False)],
+             [("a", ta[24:43], False), ("b", tb[30:31], True)],
+             [("a", ta[43:], True)]]
+    got = replay(eng, tmp_path, steps)
+    assert_logits(got["a"], cfg, w, ta, dtype)
+    assert_logits(got["b"], cfg, w, tb, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", GPU_CASES)
+def test_fast_path_sizes_in_mixed_batches(tmp_path, device, dtype):
+    cfg = fast_path_config()
+    w = write_checkpoint(tmp_path / "m", cfg)
+    reqs = {c: toks(n, seed=s) for c, n, s in
+            [("a", 150, 1), ("b", 70, 2), ("c", 101, 3), ("d", 9, 4),
+             ("e", 66, 5)]}
+    steps = mixed_plan(reqs, 3, 22, [67, 1, 1, 50, 2, 1, 33, 1, 90])
+    eng = make_engine(tmp_path / "m", device, dtype, max_tokens=352)
+    got = replay(eng, tmp_path, steps)
+    for c in reqs:
+        assert_logits(got[c], cfg, w, reqs[c], dtype, c)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_greedy_generation(tmp_path, device, dtype):
+    """LLMEngine.generate (scheduler, sampler, captured decode steps on the
+    GPU) picks the oracle's tokens; three prompts share the batch."""
+    from arks_amd.engine import SamplingParams
+
+    cfg = model_config()
+    w = write_checkpoint(tmp_path / "m", cfg)
+    prompts = [toks(19, seed=4), toks(3, seed=5), toks(34, seed=6)]
+    eng = make_engine(tmp_path / "m", device, dtype)
+    outs = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True,
+                                                temperature=0.0))
+    for p, o in zip(prompts, outs):
+        seq = list(p)
+        assert len(o) == 12
+        for tok in o:
+            logits = oracle_logits(cfg, w, seq)[-1]
+            top2 = torch.topk(logits, 2).values
+            clear = dtype == "float32" or bool(O.clear_choices(cfg, w, seq)[-1])
+            if clear and float(top2[0] - top2[1]) > (
+                    1e-3 if dtype == "float32" else 0.15):
+                assert tok == int(logits.argmax()), (len(seq), tok)
+            seq.append(tok)
+
+
+def test_preset_and_config_round_trip():
+    from arks_amd.config import PRESET_CONFIGS, HybridModelConfig
+
+    cfg = PRESET_CONFIGS["tiny-rivolix"]
+    again = HybridModelConfig.from_dict(json.loads(json.dumps(cfg.to_dict())))
+    assert again.layers == cfg.layers and again.tied_head
+    bad = cfg.to_dict()
+    bad["layers"][1]["mixer"]["kv_from"] = 2  # a later layer
+    with pytest.raises(ValueError):
+        HybridModelConfig.from_dict(bad)
+    bad["layers"][1]["mixer"]["kv_from"] = 1  # itself
+    with pytest.raises(ValueError):
+        HybridModelConfig.from_dict(bad)
+
+
+# ------------------------------------------------------- mechanisms alone
+def _dev(device):
+    return torch.device(device)
+
+
+def _rounded(x, dtype):
+    """What the op will see: the value after rounding to its row dtype."""
+    return x.to(TDT[dtype]).to(F64)
+
+
+def _i32(x, dev):
+    return torch.tensor(x, dtype=torch.int32, device=dev)
+
+
+@pytest.mark.gpu
+def test_two_map_sizes_on_the_matrix_cores():
+    """The sizes the serving presets use run the matrix-core kernels, rows
+    of prompts and single rows alike (the op says whether it took them)."""
+    from arks_amd import ops
+
+    dev = torch.device("cuda")
+    S = ops._native_seq()
+    for Dk, V in [(64, 64), (128, 128), (128, 64)]:
+        for n, single in [(40, False), (1, True)]:
+            q = torch.zeros(n, 8, Dk, dtype=torch.bfloat16, device=dev)
+            kc = torch.zeros(4, 2, 16, 2 * Dk, dtype=torch.bfloat16, device=dev)
+            vc = torch.zeros(4, 2, 16, V, dtype=torch.bfloat16, device=dev)
+            out = torch.empty(n, 8, V, dtype=torch.bfloat16, device=dev)
+            took = S.attention_masked_mfma(
+                out, q, kc, vc, _i32([[0, 1, 2, 3]], dev), _i32([40], dev),
+                _i32([0, n], dev), _i32([0] * n, dev), 0.1, None, 0.0, 0, 0,
+                1.0, single, 2)
+            assert took, (Dk, V, single)
+
+
+class MapPages:
+    """A sequence's two-map keys and shared values in pages handed out in a
+    scrambled order, and steps of rows over them through
+    ops.attention_sink_paged(maps=2)."""
+
+    def __init__(self, dev, dtype, G, Dk, V, n):
+        self.dev, self.dt = dev, TDT[dtype]
+        nblk = -(-n // 16)
+        g = torch.Generator().manual_seed(7)
+        self.table = torch.randperm(nblk + 3, generator=g)[:nblk].to(torch.int32)
+        self.k = torch.full((nblk + 3, G, 16, 2 * Dk), 9.0, dtype=self.dt, device=dev)
+        self.v = torch.full((nblk + 3, G, 16, V), 9.0, dtype=self.dt, device=dev)
+        self.len = 0
+
+    def step(self, q, k, v, scale):
+        """q [n, G, 2, R, Dk], k [n, G, 2, Dk], v [n, G, V]; rows
+        [len, len + n) join the cache; returns [n, G, 2, R, V]."""
+        from arks_amd import ops
+
+        n, G, _, R, Dk = q.shape
+        pos = torch.arange(self.len, self.len + n)
+        blk, off = self.table[pos // 16].long().to(self.dev), (pos % 16).to(self.dev)
+        self.k[blk, :, off] = k.reshape(n, G, 2 * Dk).to(self.dt).to(self.dev)
+        self.v[blk, :, off] = v.to(self.dt).to(self.dev)
+        self.len += n
+        out = ops.attention_sink_paged(
+            q.reshape(n, G * 2 * R, Dk).to(self.dt).to(self.dev).contiguous(),
+            self.k, self.v, self.table[None].to(self.dev),
+            _i32([self.len], self.dev), _i32([0, n], self.dev),
+            _i32([0] * n, self.dev), scale, False, None, False, n,
+            pos.to(self.dev), maps=2)
+        return out.double().cpu().view(n, G, 2, R, -1)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("decode", [False, True], ids=["prompt", "decoded"])
+@pytest.mark.parametrize("Dk,V", [(16, 8), (64, 64), (128, 128)],
+                         ids=["d16v8", "d64v64", "d128v128"])
+def test_one_key_wins_in_one_map_only(device, dtype, decode, Dk, V):
+    """Among hundreds of keys one gets a huge score, in ONE of the two maps:
+    that map's heads return its value, the other map's heads an average.
+    The key sits far back, on either side of a page border, at the very
+    start, and at the row itself."""
+    dev = _dev(device)
+    G, R, n = 2, 2, 300
+    i = n - 1
+    g = torch.Generator().manual_seed(5)
+    base_k = torch.randn(n, G, 2, Dk, generator=g, dtype=F64) * 0.1
+    v = _rounded(torch.randn(n, G, V, generator=g, dtype=F64), dtype)
+    e = torch.zeros(Dk, dtype=F64)
+    e[3] = 1.0
+    for hot, hot_map in [(2, 0), (0, 1), (271, 0), (272, 1), (150, 1), (i, 0)]:
+        k = base_k.clone()
+        k[hot, :, hot_map] = 40.0 * e
+        k = _rounded(k, dtype)
+        q = torch.zeros(n, G, 2, R, Dk, dtype=F64)
+        q[i] = 8.0 * e
+        want = torch.stack([
+            O.softmax_attend(q[:, :, m].reshape(n, G * R, Dk), k[:, :, m], v, 0.5)[i]
+            for m in (0, 1)], 0).view(2, G, R, V).transpose(0, 1)
+        assert torch.allclose(want[0, hot_map, 0], v[hot, 0], atol=1e-6)
+        assert not torch.allclose(want[0, 1 - hot_map, 0], v[hot, 0], atol=1e-2)
+        pg = MapPages(dev, dtype, G, Dk, V, n)
+        cut = n - 1 if decode else n - 37
+        pg.step(q[:cut], k[:cut], v[:cut], 0.5)
+        got = pg.step(q[cut:], k[cut:], v[cut:], 0.5)[-1]
+        tol = 1e-4 if dtype == "float32" else 2e-2
+        assert torch.allclose(got, want, atol=tol, rtol=tol), (hot, hot_map)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_difference_heads(device, dtype):
+    """lambda = 1 on equal maps leaves nothing but eps; lambda = 0 returns
+    map one at unit RMS; a gate far below zero closes a head; the heads of
+    one key/value head are read from the right places."""
+    from arks_amd import ops
+
+    dev = _dev(device)
+    T, H, G, V = 5, 6, 2, 12
+    g = torch.Generator().manual_seed(3)
+    a = _rounded(torch.randn(T, G, 2, H // G, V, generator=g, dtype=F64), dtype)
+    gate = _rounded(torch.randn(T, H * V + 7, generator=g, dtype=F64), dtype)
+    gate[:, 2 * V:3 * V] = -40.0
+    for lam in (0.0, 0.37, 1.0):
+        if lam == 1.0:
+            a[:, :, 1] = a[:, :, 0]
+        o = (a[:, :, 0] - lam * a[:, :, 1]).reshape(T, H, V)
+        want = (O.unit_rms(o, 1e-5) * 0.6).reshape(T, H * V) * O.sigmoid(gate[:, :H * V])
+        out = torch.zeros(T, H * V + 3, dtype=TDT[dtype], device=dev)
+        ops.diff_head_norm_gate(
+            a.reshape(T, 2 * H, V).to(TDT[dtype]).to(dev),
+            gate.to(TDT[dtype]).to(dev)[:, :H * V], lam, 1e-5, 0.6, H, G,
+            out[:, :H * V])
+        got = out.double().cpu()
+        tol = 1e-5 if dtype == "float32" else 2e-2
+        assert torch.allclose(got[:, :H * V], want, atol=tol, rtol=tol), lam
+        assert float(got[:, H * V:].abs().max()) == 0.0
+        assert float(got[:, 2 * V:3 * V].abs().max()) < 1e-12
+        if lam == 1.0:
+            assert float(got.abs().max()) < 1e-2
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("taps,dims", [(4, (8, 8)), (1, (8, 16)), (3, (5, 7))],
+                         ids=["four-taps", "one-tap", "odd"])
+def test_convolution_history_factor_and_pages(device, dtype, taps, dims):
+    """Portions of 1, 2, 9 and 1 rows of one sequence beside a second one in
+    the same steps, slots and pages filled with junk beforehand: every
+    output equals the whole-sequence convolution; q carries the factor of
+    its position (steps of the logarithm at 3, 7, 11: inside portions and
+    at their first rows) in the regrouped head order; k and v land in
+    their pages."""
+    from arks_amd import ops
+
+    dev, dt = _dev(device), TDT[dtype]
+    Dq, Vd = dims
+    H, G, M = 4, 2, 2
+    n_q, n_k, n_v = H * M * Dq, G * M * Dq, G * Vd
+    C = n_q + n_k + n_v
+    g = torch.Generator().manual_seed(4)
+    w = torch.randn(C, taps, generator=g, dtype=F64).float().double()
+    lens = {0: 13, 1: 6}
+    x = {s: _rounded(torch.randn(n, C + 5, generator=g, dtype=F64), dtype)
+         for s, n in lens.items()}
+    want = {s: O.causal_conv(x[s][:, :C], w) for s in lens}
+    state = torch.full((3, max(taps - 1, 1), C), 7.0, device=dev)
+    kc = torch.full((4, G, 16, M * Dq), 5.0, dtype=dt, device=dev)
+    vc = torch.full((4, G, 16, Vd), 5.0, dtype=dt, device=dev)
+    page = {0: 2, 1: 0}
+    slot = {0: 2, 1: 0}
+    plan = [[(0, 1), (1, 2)], [(0, 2), (1, 1)], [(0, 9)], [(1, 3), (0, 1)]]
+    at = {0: 0, 1: 0}
+    coef, every = 0.5, 4
+    tol = 1e-5 if dtype == "float32" else 3e-2
+    for step in plan:
+        rows = torch.cat([x[s][at[s]:at[s] + n] for s, n in step]).to(dt).to(dev)
+        pos = torch.cat([torch.arange(at[s], at[s] + n) for s, n in step])
+        cu = [0]
+        for _, n in step:
+            cu.append(cu[-1] + n)
+        q = ops.conv_qkv_cache(
+            rows, n_q, n_k, n_v, w.float().to(dev), w.float().t().contiguous().to(dev),
+            state if taps > 1 else None, _i32(cu, dev),
+            _i32([at[s] + n for s, n in step], dev),
+            _i32([slot[s] for s, _ in step], dev),
+            _i32(sum([[j] * n for j, (_, n) in enumerate(step)], []), dev),
+            pos.to(dev), coef, every, H, G, M, kc, vc,
+            torch.cat([page[s] * 16 + torch.arange(at[s], at[s] + n)
+                       for s, n in step]).to(dev))
+        q = q.double().cpu().view(-1, G, M, H // G, Dq)
+        r0 = 0
+        for s, n in step:
+            y = want[s][at[s]:at[s] + n]
+            f = O.query_temperature(torch.arange(at[s], at[s] + n), coef, every)
+            yq = (y[:, :n_q] * f[:, None]).view(n, G, H // G, M, Dq).transpose(2, 3)
+            assert torch.allclose(q[r0:r0 + n], yq, atol=tol, rtol=tol), (s, at[s])
+            at[s] += n
+            r0 += n
+    for s, n in lens.items():
+        gk = kc[page[s], :, :n].double().cpu().transpose(0, 1).reshape(n, n_k)
+        gv = vc[page[s], :, :n].double().cpu().transpose(0, 1).reshape(n, n_v)
+        assert torch.allclose(gk, want[s][:, n_q:n_q + n_k], atol=tol, rtol=tol)
+        assert torch.allclose(gv, want[s][:, n_q + n_k:], atol=tol, rtol=tol)
+    assert float(kc[1].float().min()) == 5.0 and float(kc[3].float().min()) == 5.0
+    assert math.isclose(float(O.query_temperature(torch.tensor([2]), coef, every)), 1.0)
+    assert float(O.query_temperature(torch.tensor([3]), coef, every)) > 1.3
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("width", [40, 64, 2056], ids=["w40", "w64", "w2056"])
+def test_residual_pair_norm(device, dtype, width):
+    from arks_amd import ops
+
+    dev, dt = _dev(device), TDT[dtype]
+    T = 7
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(T, width, generator=g, dtype=F64).float().double() * 3.0
+    y1 = _rounded(torch.randn(T, width, generator=g, dtype=F64), dtype)
+    y2 = _rounded(torch.randn(T, width, generator=g, dtype=F64), dtype)
+    s1, s2, w1, w2 = (torch.randn(width, generator=g, dtype=F64).float().double()
+                      for _ in range(4))
+    tol = 1e-5 if dtype == "float32" else 2e-2
+    for have1, have2, norms in [(True, True, 2), (True, False, 1),
+                                (False, False, 2), (False, True, 0)]:
+        xs = x.float().to(dev)
+        new = x + (y1 * s1 if have1 else 0) + (y2 * s2 if have2 else 0)
+        h1, h2 = ops.residual_pair_norm(
+            xs, y1.to(dt).to(dev) if have1 else None,
+            s1.float().to(dev) if have1 else None,
+            y2.to(dt).to(dev) if have2 else None,
+            s2.float().to(dev) if have2 else None,
+            w1.float().to(dev) if norms >= 1 else None,
+            w2.float().to(dev) if norms >= 2 else None, 1e-5, dt)
+        assert torch.allclose(xs.double().cpu(), new, atol=1e-5, rtol=1e-6)
+        for h, w in ((h1, w1), (h2, w2)):
+            if h is not None:
+                assert torch.allclose(h.double().cpu(), O.offset_norm(new, w, 1e-5),
+                                      atol=tol, rtol=tol)
+        assert (h1 is None) == (norms < 1) and (h2 is None) == (norms < 2)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_rotary_then_unit_norm(device, dtype):
+    """q and k are turned (scaled frequencies, cos and sin times the
+    factor's magnitude) and THEN brought to unit RMS; the value written
+    beside the key is the key as it came."""
+    from arks_amd import ops
+    from arks_amd.models.mixers import ramp_scaled_inv_freq
+
+    dev, dt = _dev(device), TDT[dtype]
+    rot = {"base": 100.0, "dims": 8,
+           "scaling": {"factor": 4.0, "original": 16, "fast": 4.0, "slow": 0.5}}
+    T, H, G, Dh = 6, 4, 2, 12
+    g = torch.Generator().manual_seed(9)
+    q = _rounded(torch.randn(T, H, Dh, generator=g, dtype=F64) * 3, dtype)
+    k = _rounded(torch.randn(T, G, Dh, generator=g, dtype=F64) * 0.2, dtype)
+    pos = torch.tensor([0, 1, 2, 40, 41, 1000])
+    f, mag = ramp_scaled_inv_freq(rot["base"], rot["dims"], rot["scaling"])
+    of, omag = O.ramped_freqs(rot)
+    assert torch.allclose(f.double(), of, rtol=1e-6) and math.isclose(mag, omag)
+    assert not torch.allclose(of, O.ramped_freqs({"base": 100.0, "dims": 8})[0])
+    kc = torch.zeros(70, G, 16, Dh, dtype=dt, device=dev)
+    vc = torch.zeros(70, G, 16, Dh, dtype=dt, device=dev)
+    kk = k.to(dt).to(dev)
+    qo = ops.qk_norm_rope_cache(
+        q.to(dt).to(dev), kk, kk, None, None, 1e-5, pos.to(dev), f.to(dev), None,
+        kc, vc, pos.to(dev), False, mag, True)
+    tol = 1e-5 if dtype == "float32" else 2e-2
+    want_q = O.unit_rms(O.rotate_half(q, pos, rot), 1e-5)
+    want_k = O.unit_rms(O.rotate_half(k, pos, rot), 1e-5)
+    assert torch.allclose(qo.double().cpu(), want_q, atol=tol, rtol=tol)
+    got_k = kc.double().cpu()[pos // 16, :, pos % 16]
+    got_v = vc.double().cpu()[pos // 16, :, pos % 16]
+    assert torch.allclose(got_k, want_k, atol=tol, rtol=tol)
+    assert torch.equal(got_v, k)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_scores_scale_the_experts_input(device, dtype):
+    """Router rows made so that the choice is known: the chosen scores are
+    the plain sigmoids (not renormalised), and an expert's result is
+    expert(score * h), which differs from score * expert(h)."""
+    from arks_amd import ops
+
+    dev, dt = _dev(device), TDT[dtype]
+    z = torch.tensor([[3.0, -1.0, 0.5, 2.0, -4.0], [-2.0, -3.0, -1.0, -5.0, -2.5],
+                      [0.1, 0.0, -0.1, -0.2, 7.0]])
+    wts, ids, mat = ops.moe_route_grouped(z.to(dev), 2, 1, 1, "sigmoid", False,
+                                          matrix=True)
+    assert ids.cpu().tolist() == [[0, 3], [2, 0], [4, 0]]
+    s = torch.sigmoid(z)
+    assert torch.allclose(wts.cpu(), torch.gather(s, 1, ids.cpu().long()), atol=1e-6)
+    dense = torch.zeros_like(s).scatter(1, ids.cpu().long(), wts.cpu())
+    assert torch.allclose(mat.cpu(), dense, atol=1e-6)
+    E, ff, sff, W = 5, 8, 16, 24
+    g = torch.Generator().manual_seed(10)
+    w = {f"e{e}.{n}": torch.randn(*(shape), generator=g, dtype=F64) * 0.5
+         for e in range(E) for n, shape in
+         (("gate", (ff, W)), ("up", (ff, W)), ("down", (W, ff)))}
+    w.update({"shared.gate": torch.randn(sff, W, generator=g, dtype=F64) * 0.5,
+              "shared.up": torch.randn(sff, W, generator=g, dtype=F64) * 0.5})
+    h = _rounded(torch.randn(3, W, generator=g, dtype=F64), dtype)
+    gu = torch.cat([torch.cat([h @ w[f"e{e}.gate"].T, h @ w[f"e{e}.up"].T], 1)
+                    for e in range(E)]
+                   + [h @ w["shared.gate"].T, h @ w["shared.up"].T], 1)
+    gu = _rounded(gu, dtype)
+    act = ops.moe_glu_scaled(gu.to(dt).to(dev), mat, E, ff, sff).double().cpu()
+    tol = 1e-5 if dtype == "float32" else 3e-2
+    for t in range(3):
+        for e in range(E):
+            ge, ue = gu[t, e * 2 * ff:e * 2 * ff + ff], gu[t, e * 2 * ff + ff:(e + 1) * 2 * ff]
+            sc = float(dense[t, e])
+            want = O.silu(sc * ge) * (sc * ue)
+            assert torch.allclose(act[t, e * ff:(e + 1) * ff], want, atol=tol, rtol=tol)
+            if sc == 0.0:
+                assert float(act[t, e * ff:(e + 1) * ff].abs().max()) == 0.0
+            else:
+                assert not torch.allclose(want, sc * O.silu(ge) * ue, atol=1e-3)
+        sh = gu[t, E * 2 * ff:]
+        assert torch.allclose(act[t, E * ff:], O.silu(sh[:sff]) * sh[sff:],
+                              atol=tol, rtol=tol)
