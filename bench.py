@@ -52,14 +52,18 @@ def parse_args():
     # random-init path the serving bench uses).
     # NOT the headline either: prefill and decode throughput of a layer-list
     # design (--design) at real layer sizes beside the closest llama-family
-    # model cut to the same width and depth, one JSON line per model and
-    # phase. --design-only NAME runs one of the two (profiling).
+    # model cut to the same width and depth (for rivolix, whose feed-forward
+    # is routed experts beside a shared one: a Qwen2-MoE-shaped model of the
+    # same width, depth, head and expert sizes, "moe"), one JSON line per
+    # model and phase. --design-only NAME runs one of the two (profiling).
     p.add_argument("--design-bench", action="store_true")
     p.add_argument("--design-only",
-                   choices=["gagorax", "fusolix", "legalix", "llama"],
+                   choices=["gagorax", "fusolix", "legalix", "rivolix", "llama",
+                            "moe"],
                    default=None)
     # which layer-list design --design-bench measures beside llama
-    p.add_argument("--design", choices=["gagorax", "fusolix", "legalix"],
+    p.add_argument("--design",
+                   choices=["gagorax", "fusolix", "legalix", "rivolix"],
                    default="gagorax")
     p.add_argument("--cold-start", action="store_true")
     p.add_argument("--ckpt-dir", default="/tmp/arks_ckpt")
@@ -131,8 +135,9 @@ def run_cold_start(args):
 
 
 def run_design_bench(args):
-    """A layer-list design (--design: Gagorax, Fusolix or Legalix, 8 blocks at the
-    sizes of an 8B model) against llama-3-8b cut to 8 layers: prefill
+    """A layer-list design (--design: Gagorax, Fusolix, Legalix or Rivolix, 8
+    blocks at the sizes of an 8B model) against llama-3-8b cut to 8 layers
+    (Rivolix: against a Qwen2-MoE-shaped model of equal sizes): prefill
     tokens/s for one long prompt and for a batch of prompts, decode tokens/s
     for a batch at a fixed context. Random weights, synthetic tokens, one
     GPU."""
@@ -145,6 +150,16 @@ def run_design_bench(args):
         PRESET_CONFIGS["llama-3-8b"], num_hidden_layers=8)
     use_gpu = torch.cuda.is_available()
     models = {args.design: args.design + "-8b-slice", "llama": "llama-3-8b-8l"}
+    if args.design == "rivolix":
+        # the same expert layout in the llama family: 16 experts of ff 3584,
+        # 4 per row, a shared expert of ff 3584, 32/8 heads x 128
+        PRESET_CONFIGS["qwen2moe-8b-8l"] = dataclasses.replace(
+            PRESET_CONFIGS["llama-3-8b"], architecture="Qwen2MoeForCausalLM",
+            num_hidden_layers=8, vocab_size=32000, num_local_experts=16,
+            num_experts_per_tok=4, moe_intermediate_size=3584,
+            shared_expert_intermediate_size=3584, norm_topk_prob=False,
+            attention_bias=True, tie_word_embeddings=True)
+        models = {"rivolix": "rivolix-8b-slice", "moe": "qwen2moe-8b-8l"}
     prefills = [(1, 8192), (8, 2048), (32, 128)]  # (prompts, tokens each)
     dec_batch, dec_ctx = args.batch, args.input_len
     for key, preset in models.items():
