@@ -219,8 +219,9 @@ __global__ __launch_bounds__(256) void conv_qkv_cache_kernel(
 
 // bf16 rows, 8 channels per thread (a piece never crosses a head, a map or
 // the q | k | v borders: dim, kdim, vdim, n_q, n_k all multiples of 8) and
-// QKV_RPT consecutive rows per block with the thread's taps in registers;
-// w_t [taps, C] is a transposed copy of the taps.
+// rpt consecutive rows per block (QKV_RPT in long steps, fewer in short
+// ones so that the launch still fills the chip) with the thread's taps in
+// registers; w_t [taps, C] is a transposed copy of the taps.
 constexpr int QKV_RPT = 8;
 constexpr int QKV_MAX_TAPS = QKV_MAX_HIST + 1;
 
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(256) void conv_qkv_cache_vec8_kernel(
     const int* __restrict__ slots, const int* __restrict__ token_seq,
     const int64_t* __restrict__ positions, bf16* __restrict__ k_cache,
     bf16* __restrict__ v_cache, const int64_t* __restrict__ slot_mapping,
-    int T, QkvConvArgs a) {
+    int T, int rpt, QkvConvArgs a) {
   const int C = a.n_q + a.n_k + a.n_v;
   const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
   if (c >= C) return;
@@ -260,8 +261,8 @@ __global__ __launch_bounds__(256) void conv_qkv_cache_vec8_kernel(
     g = (c - a.n_q - a.n_k) / a.vdim;
     dst0 = (c - a.n_q - a.n_k) % a.vdim;
   }
-  const int t_end = min(T, (int)(blockIdx.x + 1) * QKV_RPT);
-  for (int t = blockIdx.x * QKV_RPT; t < t_end; ++t) {
+  const int t_end = min(T, (int)(blockIdx.x + 1) * rpt);
+  for (int t = blockIdx.x * rpt; t < t_end; ++t) {
     const SeqRow r = seq_row(t, token_seq, cu, seq_lens, slots);
     const int i = t - r.first_row;
     const bool has_state = r.start > 0 && r.slot >= 0 && a.taps > 1;
@@ -394,6 +395,47 @@ __global__ __launch_bounds__(256) void diff_head_norm_gate_kernel(
   }
 }
 
+// bf16, 8 values per lane: a head is V / 8 neighbouring lanes (a power of
+// two, at most 64), so a wave holds 512 / V heads and reduces inside each.
+__global__ __launch_bounds__(256) void diff_head_norm_gate_vec8_kernel(
+    bf16* __restrict__ out, int64_t ldo, const bf16* __restrict__ a,
+    const bf16* __restrict__ gate, int64_t ldg, float lam, float eps,
+    float mult, int64_t n_heads, int H, int G, int V) {
+  const int L = V / 8;  // lanes per head
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) / L;
+  const int d = (threadIdx.x % L) * 8;
+  const bool live = idx < n_heads;
+  const int64_t t = live ? idx / H : 0;
+  const int h = live ? (int)(idx % H) : 0;
+  const int R = H / G;
+  const int g = h / R, i = h % R;
+  float o[8];
+  float ss = 0.f;
+  if (live) {
+    const ushort8 u1 = *reinterpret_cast<const ushort8*>(
+        a + (((t * G + g) * 2 + 0) * R + i) * V + d);
+    const ushort8 u2 = *reinterpret_cast<const ushort8*>(
+        a + (((t * G + g) * 2 + 1) * R + i) * V + d);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      o[e] = bf16_bits_to_float(u1[e]) - lam * bf16_bits_to_float(u2[e]);
+      ss += o[e] * o[e];
+    }
+  }
+  for (int off = L / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, WAVE_SIZE);
+  if (!live) return;
+  const float f = mult / sqrtf(ss / (float)V + eps);
+  const ushort8 gv =
+      *reinterpret_cast<const ushort8*>(gate + t * ldg + (int64_t)h * V + d);
+  ushort8 r;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float z = bf16_bits_to_float(gv[e]);
+    r[e] = float_to_bf16_bits(o[e] * f / (1.f + __expf(-z)));
+  }
+  *reinterpret_cast<ushort8*>(out + t * ldo + (int64_t)h * V + d) = r;
+}
+
 // ------------------------------------------------------- expert activation
 template <typename AT>
 __global__ __launch_bounds__(256) void moe_glu_scaled_kernel(
@@ -508,16 +550,21 @@ extern "C" int arks_seq_conv_qkv_cache(
   const bool vec8 = !act_f32 && w_t && ldp % 8 == 0 &&
                     ((uintptr_t)p % 16) == 0 && a.dim % 8 == 0 &&
                     a.kdim % 8 == 0 && a.vdim % 8 == 0;
+  // rows per block: as many as leave about 1024 blocks
+  const int cb8 = (C / 8 + 255) / 256;
+  int rpt = (int)(((int64_t)T * cb8) / 1024);
+  rpt = rpt < 1 ? 1 : (rpt > QKV_RPT ? QKV_RPT : rpt);
   SEQ_DISPATCH_ACT(act_f32, {
     if (vec8)
       hipLaunchKernelGGL(conv_qkv_cache_vec8_kernel,
-                         dim3((T + QKV_RPT - 1) / QKV_RPT, (C / 8 + 255) / 256),
+                         dim3((T + rpt - 1) / rpt, cb8),
                          dim3(256), 0, stream, (bf16*)qo, (const bf16*)p, ldp,
                          (const float*)w_t, (const float*)state,
                          (const int*)cu, (const int*)seq_lens,
                          (const int*)slots, (const int*)token_seq,
                          (const int64_t*)positions, (bf16*)k_cache,
-                         (bf16*)v_cache, (const int64_t*)slot_mapping, T, a);
+                         (bf16*)v_cache, (const int64_t*)slot_mapping, T, rpt,
+                         a);
     else
       hipLaunchKernelGGL((conv_qkv_cache_kernel<AT>), dim3(T, cb), dim3(256),
                          0, stream, (AT*)qo, (const AT*)p, ldp,
@@ -542,6 +589,17 @@ extern "C" int arks_seq_diff_head_norm_gate(
   if (V > 64 * DIFF_VPT) return 1;
   if (T == 0) return 0;
   const int64_t n = (int64_t)T * H;
+  const int L = V / 8;
+  if (!act_f32 && V % 8 == 0 && L <= 64 && (L & (L - 1)) == 0 &&
+      ldo % 8 == 0 && ldg % 8 == 0 && ((uintptr_t)out & 15) == 0 &&
+      ((uintptr_t)gate & 15) == 0 && ((uintptr_t)a & 15) == 0) {
+    const int64_t threads = n * L;
+    hipLaunchKernelGGL(diff_head_norm_gate_vec8_kernel,
+                       dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                       stream, (bf16*)out, ldo, (const bf16*)a,
+                       (const bf16*)gate, ldg, lam, eps, mult, n, H, G, V);
+    return 0;
+  }
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
       (diff_head_norm_gate_kernel<AT>), dim3((unsigned)((n + 3) / 4)),
       dim3(256), 0, stream, (AT*)out, ldo, (const AT*)a, (const AT*)gate, ldg,

@@ -512,24 +512,26 @@ def test_one_key_wins_in_one_map_only(device, dtype, decode, Dk, V):
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
-def test_difference_heads(device, dtype):
+@pytest.mark.parametrize("V", [12, 64, 128], ids=["v12", "v64", "v128"])
+def test_difference_heads(device, dtype, V):
     """lambda = 1 on equal maps leaves nothing but eps; lambda = 0 returns
     map one at unit RMS; a gate far below zero closes a head; the heads of
     one key/value head are read from the right places."""
     from arks_amd import ops
 
     dev = _dev(device)
-    T, H, G, V = 5, 6, 2, 12
+    T, H, G = 5, 6, 2
+    pad = 8 if V % 8 == 0 else 7  # rows the 16-byte kernels can take, or not
     g = torch.Generator().manual_seed(3)
     a = _rounded(torch.randn(T, G, 2, H // G, V, generator=g, dtype=F64), dtype)
-    gate = _rounded(torch.randn(T, H * V + 7, generator=g, dtype=F64), dtype)
+    gate = _rounded(torch.randn(T, H * V + pad, generator=g, dtype=F64), dtype)
     gate[:, 2 * V:3 * V] = -40.0
     for lam in (0.0, 0.37, 1.0):
         if lam == 1.0:
             a[:, :, 1] = a[:, :, 0]
         o = (a[:, :, 0] - lam * a[:, :, 1]).reshape(T, H, V)
         want = (O.unit_rms(o, 1e-5) * 0.6).reshape(T, H * V) * O.sigmoid(gate[:, :H * V])
-        out = torch.zeros(T, H * V + 3, dtype=TDT[dtype], device=dev)
+        out = torch.zeros(T, H * V + pad, dtype=TDT[dtype], device=dev)
         ops.diff_head_norm_gate(
             a.reshape(T, 2 * H, V).to(TDT[dtype]).to(dev),
             gate.to(TDT[dtype]).to(dev)[:, :H * V], lam, 1e-5, 0.6, H, G,
