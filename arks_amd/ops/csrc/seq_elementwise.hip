@@ -366,6 +366,128 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
   }
 }
 
+// bf16 rows, half-split pairs, values stored plain, D / 8 lanes per head
+// slot (a power of two, at most 64; V <= D), 8 dims per lane with 16-byte
+// accesses: the same work as qk_norm_rope_cache_kernel, one block per row,
+// the row's cos / sin (times rot_mag) once in LDS. A pair's two dims sit
+// n_rot apart, i.e. n_rot / 8 lanes apart (n_rot % 8 == 0): the partner's
+// values come by shuffle. Sums of squares are reduced inside a head's lanes.
+__global__ __launch_bounds__(256) void qk_norm_rope_cache_vec8_kernel(
+    bf16* __restrict__ qo, const bf16* __restrict__ q,
+    const bf16* __restrict__ k, const bf16* __restrict__ v, int64_t ldq,
+    int64_t ldk, int64_t ldv, const float* __restrict__ qw,
+    const float* __restrict__ kw, float eps,
+    const int64_t* __restrict__ positions, const float* __restrict__ freq_qk,
+    int n_rot, bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
+    const int64_t* __restrict__ slot_mapping, int H, int G, int D, int V,
+    int block_size, float rot_mag, int norm_after) {
+  __shared__ float cs_qk[ROPE_MAX_PAIRS][2];
+  const int t = blockIdx.x;
+  const float pos = (float)positions[t];
+  for (int i = threadIdx.x; i < n_rot; i += 256) {
+    float sn, cs;
+    sincosf(pos * freq_qk[i], &sn, &cs);
+    cs_qk[i][0] = cs * rot_mag;
+    cs_qk[i][1] = sn * rot_mag;
+  }
+  __syncthreads();
+  const int L = D / 8;
+  const int sub = threadIdx.x % L;          // lane inside the head
+  const int d0 = sub * 8;
+  const int per_pass = 256 / L;
+  const int lane = threadIdx.x % WAVE_SIZE;
+  const int hop = n_rot / 8;                // lanes between a pair's dims
+  const int64_t slot = slot_mapping[t];
+  const int n_slots = H + 2 * G;
+  for (int hs0 = 0; hs0 < n_slots; hs0 += per_pass) {
+    const int hs = hs0 + threadIdx.x / L;
+    const bool live = hs < n_slots;
+    const bf16* src = nullptr;
+    bf16* dst = nullptr;
+    const float* nw = nullptr;
+    bool is_v = false;
+    if (live) {
+      if (hs < H) {
+        src = q + (int64_t)t * ldq + (int64_t)hs * D;
+        dst = qo + ((int64_t)t * H + hs) * D;
+        nw = qw;
+      } else if (slot >= 0) {
+        const int64_t blk = slot / block_size, off = slot % block_size;
+        if (hs < H + G) {
+          const int g = hs - H;
+          src = k + (int64_t)t * ldk + (int64_t)g * D;
+          dst = k_cache + ((blk * G + g) * block_size + off) * D;
+          nw = kw;
+        } else {
+          const int g = hs - H - G;
+          is_v = true;
+          if (d0 < V) {
+            src = v + (int64_t)t * ldv + (int64_t)g * V;
+            dst = v_cache + ((blk * G + g) * block_size + off) * V;
+          }
+        }
+      }
+    }
+    float x[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = 0.f;
+    if (src) {
+      const ushort8 u = *reinterpret_cast<const ushort8*>(src + d0);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = bf16_bits_to_float(u[e]);
+    }
+    if (is_v) {  // values pass as they are (every lane still joins the shuffles)
+      if (src) {
+        const ushort8 u = *reinterpret_cast<const ushort8*>(src + d0);
+        *reinterpret_cast<ushort8*>(dst + d0) = u;
+      }
+      src = nullptr;
+    }
+    if (qw != nullptr) {  // norm with a weight in front of the turn
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+      for (int off = L / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, WAVE_SIZE);
+      const float rstd = 1.f / sqrtf(ss / (float)D + eps);
+      if (nw) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] *= rstd * nw[d0 + e];
+      }
+    }
+    if (n_rot > 0) {
+      const bool first = d0 < n_rot, second = !first && d0 < 2 * n_rot;
+      const int partner = first ? lane + hop : lane - hop;
+      float y[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        y[e] = __shfl(x[e], (first || second) ? partner : lane, WAVE_SIZE);
+      if (first || second) {
+        const int i0 = first ? d0 : d0 - n_rot;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float c = cs_qk[i0 + e][0], sn = cs_qk[i0 + e][1];
+          x[e] = first ? x[e] * c - y[e] * sn : x[e] * c + y[e] * sn;
+        }
+      }
+    }
+    if (norm_after) {
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+      for (int off = L / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, WAVE_SIZE);
+      const float rstd = 1.f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] *= rstd;
+    }
+    if (src) {
+      ushort8 o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = float_to_bf16_bits(x[e]);
+      *reinterpret_cast<ushort8*>(dst + d0) = o;
+    }
+  }
+}
+
 // Turn every head row of out [T, H, V] back by its row's position: pair m
 // by -pos * freq[m] (the cache holds values turned forward by their own
 // positions, so the weighted sum comes out in the query's frame). One block
@@ -482,6 +604,21 @@ extern "C" int arks_seq_qk_norm_rope_cache(
     float rot_mag, int norm_after, hipStream_t stream) {
   if (n_rot > ROPE_MAX_PAIRS || n_vrot > ROPE_MAX_PAIRS) return 1;
   if (T == 0) return 0;
+  const int L = D / 8;
+  if (!act_f32 && !interleaved && n_vrot == 0 && D % 8 == 0 && V % 8 == 0 &&
+      V <= D && L <= 64 && (L & (L - 1)) == 0 && n_rot % 8 == 0 &&
+      ldq % 8 == 0 && ldk % 8 == 0 && ldv % 8 == 0 &&
+      (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)qo |
+        (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0) {
+    hipLaunchKernelGGL(
+        qk_norm_rope_cache_vec8_kernel, dim3(T), dim3(256), 0, stream,
+        (bf16*)qo, (const bf16*)q, (const bf16*)k, (const bf16*)v, ldq, ldk,
+        ldv, (const float*)qw, (const float*)kw, eps,
+        (const int64_t*)positions, (const float*)freq_qk, n_rot,
+        (bf16*)k_cache, (bf16*)v_cache, (const int64_t*)slot_mapping, H, G, D,
+        V, block_size, rot_mag, norm_after);
+    return 0;
+  }
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
       (qk_norm_rope_cache_kernel<AT>), dim3(T), dim3(256), 0, stream,
       (AT*)qo, (const AT*)q, (const AT*)k, (const AT*)v, ldq, ldk, ldv,

@@ -100,7 +100,9 @@ void attn_masked_tile_kernel(
     seq_idx = token_seq[blockIdx.y];
     p0 = blockIdx.y - cu[seq_idx];
   } else {
-    int left = blockIdx.y;
+    // the last tiles of a sequence see the most keys: they start first, so
+    // the launch ends on short tiles
+    int left = gridDim.y - 1 - blockIdx.y;
     for (int s = 0; s < num_seqs; ++s) {
       const int n = (cu[s + 1] - cu[s] + PPT - 1) / PPT;
       if (left < n) {
