@@ -379,7 +379,7 @@ def _rivolix_preset(width, vocab, pattern, heads, kv_heads, dim, vdim, taps,
     for i, ch in enumerate(pattern):
         if ch in "ds":
             m = {"heads": heads, "kv_heads": kv_heads, "dim": dim,
-                 "vdim": vdim, "conv": taps, "diff": 0.3,
+                 "vdim": vdim, "conv": taps, "diff": 0.2,
                  "q_temp": {"coef": 0.1, "every": 1024},
                  "scale": dim ** -0.5}
             if ch == "s":
@@ -391,9 +391,9 @@ def _rivolix_preset(width, vocab, pattern, heads, kv_heads, dim, vdim, taps,
             spec = {"type": "attention_2", "mixer": {
                 "heads": k_heads, "kv_heads": k_kv_heads, "dim": k_dim,
                 "vdim": k_dim, "scale": k_dim ** -0.5,
-                "rot": {"base": 500000.0, "dims": k_dim // 2,
-                        "scaling": {"factor": 8.0, "original": 8192,
-                                    "fast": 32.0, "slow": 1.0}}}}
+                "rot": {"base": 1000000.0, "dims": k_dim // 2,
+                        "scaling": {"factor": 4.0, "original": 4096,
+                                    "fast": 16.0, "slow": 2.0}}}}
         spec["mlp"] = {"kind": "moe", "expert": {"ff": expert_ff},
                        "router": {"experts": experts, "top": top},
                        "shared": {"ff": shared_ff} if shared_ff else None}
@@ -706,7 +706,7 @@ PRESET_CONFIGS: dict[str, ModelConfig] = {
         4096, 32000, "dskddskd", 16, 4, 128, 128, 4, 32, 8, 128, 16, 4, 3584,
         3584),
     "tiny-rivolix": _rivolix_preset(
-        128, 512, "dsk", 4, 2, 16, 24, 3, 6, 2, 32, 8, 2, 48, 80),
+        128, 512, "dsk", 6, 2, 16, 24, 4, 4, 2, 32, 8, 2, 48, 80),
     "tiny-gpu": ModelConfig(  # GPU-test-sized (head_dim 128 kernels)
         architecture="Qwen2ForCausalLM",
         vocab_size=2048,

@@ -397,7 +397,7 @@ def test_preset_and_config_round_trip():
     cfg = PRESET_CONFIGS["tiny-rivolix"]
     again = HybridModelConfig.from_dict(json.loads(json.dumps(cfg.to_dict())))
     assert again.layers == cfg.layers and again.tied_head
-    bad = cfg.to_dict()
+    bad = json.loads(json.dumps(cfg.to_dict()))  # the preset stays as it is
     bad["layers"][1]["mixer"]["kv_from"] = 2  # a later layer
     with pytest.raises(ValueError):
         HybridModelConfig.from_dict(bad)
@@ -575,7 +575,7 @@ def test_convolution_history_factor_and_pages(device, dtype, taps, dims):
     slot = {0: 2, 1: 0}
     plan = [[(0, 1), (1, 2)], [(0, 2), (1, 1)], [(0, 9)], [(1, 3), (0, 1)]]
     at = {0: 0, 1: 0}
-    coef, every = 0.5, 4
+    coef, every = 0.6, 4
     tol = 1e-5 if dtype == "float32" else 3e-2
     for step in plan:
         rows = torch.cat([x[s][at[s]:at[s] + n] for s, n in step]).to(dt).to(dev)

@@ -500,7 +500,7 @@ def test_cli_flags_map_to_engine_config():
 
 
 @pytest.mark.parametrize("preset", ["tiny-gagorax", "tiny-fusolix",
-                                    "tiny-legalix"])
+                                    "tiny-legalix", "tiny-rivolix"])
 def test_layer_list_preset_serves_completions(preset):
     """A layer-list model (recurrent state slots, no prefix reuse) behind
     the same HTTP front: a completion and a streamed chat, twice, so slots
