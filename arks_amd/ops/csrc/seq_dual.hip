@@ -140,7 +140,8 @@ __global__ __launch_bounds__(256) void residual_pair_norm_vec8_kernel(
 }
 
 // ----------------------------------------------------------- convolution
-constexpr int QKV_MAX_HIST = 8;  // taps - 1
+constexpr int QKV_MAX_HIST = 31;     // taps - 1, general kernels
+constexpr int QKV_VEC_MAX_TAPS = 9;  // taps the vectorised kernel holds
 
 struct QkvConvArgs {
   int n_q, n_k, n_v;       // channels of each kind, in this order
@@ -223,7 +224,7 @@ __global__ __launch_bounds__(256) void conv_qkv_cache_kernel(
 // ones so that the launch still fills the chip) with the thread's taps in
 // registers; w_t [taps, C] is a transposed copy of the taps.
 constexpr int QKV_RPT = 8;
-constexpr int QKV_MAX_TAPS = QKV_MAX_HIST + 1;
+constexpr int QKV_MAX_TAPS = QKV_VEC_MAX_TAPS;
 
 __global__ __launch_bounds__(256) void conv_qkv_cache_vec8_kernel(
     bf16* __restrict__ qo, const bf16* __restrict__ p, int64_t ldp,
@@ -547,7 +548,8 @@ extern "C" int arks_seq_conv_qkv_cache(
   a.temp_coef = temp_coef; a.temp_every = temp_every;
   const int C = n_q + n_k + n_v;
   const int cb = (C + 255) / 256;
-  const bool vec8 = !act_f32 && w_t && ldp % 8 == 0 &&
+  const bool vec8 = !act_f32 && w_t && taps <= QKV_VEC_MAX_TAPS &&
+                    ldp % 8 == 0 &&
                     ((uintptr_t)p % 16) == 0 && a.dim % 8 == 0 &&
                     a.kdim % 8 == 0 && a.vdim % 8 == 0;
   // rows per block: as many as leave about 1024 blocks

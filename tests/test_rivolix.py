@@ -259,6 +259,7 @@ OTHER_SIZES = {
                                  K(heads=3, kv_heads=3, dim=8, rot_dims=8)]),
     "no-history": dict(layers=[D(conv=1), D(conv=1, kv_from=0)]),
     "eight-taps": dict(layers=[D(conv=8), D(conv=8, kv_from=0)]),
+    "twelve-taps": dict(layers=[D(conv=12, dim=16, vdim=16)]),
     "no-difference": dict(layers=[D(diff=0.0)]),
     "large-difference": dict(layers=[D(diff=0.8)]),
     "factor-every-position": dict(layers=[D(every=1, coef=0.9)]),
@@ -328,6 +329,25 @@ def test_fast_path_sizes(tmp_path, device, dtype):
     plan = [t[:130], t[130:131], t[131:197], t[197:198], t[198:199],
             t[199:201], t[201:]]
     assert len(plan[-1]) > 120
+    got = replay(eng, tmp_path, [[("a", p, False)] for p in plan])["a"]
+    assert_logits(got, cfg, w, t, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", GPU_CASES)
+def test_key_valued_head_sizes(tmp_path, device, dtype):
+    """Every head size the matrix-core kernels of plain causal attention are
+    built for, with the vectorised turn-and-norm kernel where the size
+    allows it (96 does not), over a prompt, single rows and a second portion."""
+    cfg = O.make_config(
+        [K(heads=4, kv_heads=2, dim=32, rot_dims=16, mlp=None),
+         K(heads=2, kv_heads=1, dim=96, rot_dims=32, mlp=None),
+         K(heads=2, kv_heads=2, dim=256, rot_dims=256, mlp=None),
+         K(heads=4, kv_heads=1, dim=64, rot_dims=0, mlp=MOE(top=6))],
+        width=64)
+    w = write_checkpoint(tmp_path / "m", cfg)
+    t = toks(180, seed=12)
+    eng = make_engine(tmp_path / "m", device, dtype, max_tokens=256)
+    plan = [t[:100], t[100:101], t[101:102], t[102:170], t[170:]]
     got = replay(eng, tmp_path, [[("a", p, False)] for p in plan])["a"]
     assert_logits(got, cfg, w, t, dtype)
 
@@ -477,8 +497,12 @@ class MapPages:
 
 @pytest.mark.parametrize("device,dtype", CASES)
 @pytest.mark.parametrize("decode", [False, True], ids=["prompt", "decoded"])
-@pytest.mark.parametrize("Dk,V", [(16, 8), (64, 64), (128, 128)],
-                         ids=["d16v8", "d64v64", "d128v128"])
+@pytest.mark.parametrize("Dk,V", [(16, 8), (64, 64), (128, 128), (128, 64),
+                                  (96, 96), (96, 64), (64, 32), (192, 128),
+                                  (32, 80)],
+                         ids=["d16v8", "d64v64", "d128v128", "d128v64",
+                              "d96v96", "d96v64", "d64v32", "d192v128",
+                              "d32v80"])
 def test_one_key_wins_in_one_map_only(device, dtype, decode, Dk, V):
     """Among hundreds of keys one gets a huge score, in ONE of the two maps:
     that map's heads return its value, the other map's heads an average.
