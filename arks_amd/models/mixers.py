@@ -807,6 +807,24 @@ class DiffAttention(SplitMixer):
             out["conv"] = ("slot", (self.taps - 1, self.ch), torch.float32)
         return out
 
+    def _prompt_tiles(self, batch: ForwardBatch, q):
+        """Work lists of the prefill kernels for a step that holds prompt
+        portions (host-built once per step and head layout); None where the
+        masked or general kernels run: steps whose longest portion does not
+        fill a 256-row tile (the masked tiles are as fast there), captured
+        graphs, float32, CPU, head sizes those kernels are not built for."""
+        if (not q.is_cuda or q.dtype != torch.bfloat16 or self.D != self.V
+                or self.D not in ops.PREFILL_MAP_DIMS or not ops.use_ladder_maps
+                or batch.kv_lens_list is None
+                or batch.max_q_len < ops.EXTEND2_QTILE):
+            return None
+        key = ("maps", self.H * self.MAPS, self.D)
+        if key not in batch.tile_cache:
+            batch.tile_cache[key] = ops.build_extend_tiles(
+                batch.seq_lens_list, batch.kv_lens_list, False, q.device,
+                num_q_heads=self.H * self.MAPS, flash_decode=False)
+        return batch.tile_cache[key]
+
     def core(self, p, batch: ForwardBatch, cache: dict, out, out_scale) -> None:
         assert out_scale == 1.0
         T = p.shape[0]
@@ -817,10 +835,20 @@ class DiffAttention(SplitMixer):
             batch.state_slots, batch.token_seq, batch.positions,
             self.temp_coef, self.temp_every, H, G, M, cache["k"], cache["v"],
             batch.slot_mapping)
-        a = ops.attention_sink_paged(
-            q.view(T, H * M, D), cache["k"], cache["v"], batch.block_tables,
-            batch.seq_lens, batch.cu_seqlens, batch.token_seq, self.scale,
-            False, None, False, batch.max_q_len, batch.positions, maps=M)
+        q = q.view(T, H * M, D)
+        tiles = self._prompt_tiles(batch, q)
+        if tiles is not None:
+            # steps with prompt portions: the framework's work-sorted
+            # prefill kernels (256-row ladder, 64-row) read the two-map rows
+            a = ops.attention_extend_paged(
+                q, cache["k"], cache["v"], batch.block_tables, batch.seq_lens,
+                batch.cu_seqlens, None, self.scale, tiles=tiles,
+                native=ops.seq_extension(), maps=M)
+        else:
+            a = ops.attention_sink_paged(
+                q, cache["k"], cache["v"], batch.block_tables, batch.seq_lens,
+                batch.cu_seqlens, batch.token_seq, self.scale, False, None,
+                False, batch.max_q_len, batch.positions, maps=M)
         ops.diff_head_norm_gate(a, p[:, self.ch:self.ch + H * V], self.lam,
                                 self.eps, 1.0 - self.diff, H, G, out)
 

@@ -232,7 +232,7 @@ def build_extend_tiles(q_lens: list[int], kv_lens: list[int] | None,
 def attention_extend_paged(
     q, k_cache, v_cache, block_tables, kv_lens, cu_seqlens_q,
     q_lens: list[int], scale: float, window: int = 0, tiles=None,
-    sink: bool = False, native=None,
+    sink: bool = False, native=None, maps: int = 1,
 ):
     """Causal attention of packed NEW tokens over each sequence's full paged
     KV history (cached prefix + new tokens already written by
@@ -241,7 +241,10 @@ def attention_extend_paged(
     D2H sync); kv_lens is the device int32 total kv length per seq.
     window > 0 = sliding-window attention. sink: every softmax also holds a
     value-less key of score 0. native: the extension whose build of these
-    kernels runs (default: arks_amd_C).
+    kernels runs (default: arks_amd_C). maps M > 1: a key row of the cache
+    holds M keys side by side that share the row's value (k_cache [pages, G,
+    16, M*D]); q has G*M groups of heads, group g*M + m reads key m of head
+    g (tiles built without the flash-decode rows).
 
     Dispatch: big chunks run the 8-wave 32x32-MFMA ladder kernel
     (attn_extend2.hip, 256-row q tiles); small chunks and fp8-KV runs use
@@ -268,7 +271,7 @@ def attention_extend_paged(
                 ws = q.new_empty(0, dtype=torch.float32)
             C.attention_extend_paged2(
                 out, q, k_cache, v_cache, block_tables, kv_lens, cu_seqlens_q,
-                t256, ws, scale, window, sink,
+                t256, ws, scale, window, sink, maps,
             )
             if ctab.numel():
                 C.attention_extend2_combine(
@@ -277,9 +280,10 @@ def attention_extend_paged(
         if t64.numel():
             C.attention_extend_paged(
                 out, q, k_cache, v_cache, block_tables, kv_lens, cu_seqlens_q,
-                t64, scale, window, sink,
+                t64, scale, window, sink, maps,
             )
         if drows is not None:
+            assert maps == 1, "single rows of a two-map cache: no flash-decode"
             dq = q[drows].contiguous()
             dout = attention_decode_paged(
                 dq, k_cache, v_cache,
@@ -749,6 +753,16 @@ def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
 
 
 use_masked_mfma = True  # tests switch it off to compare both paths
+# prompt portions over two-map key rows: the work-sorted prefill kernels
+# (head sizes of the 256-row ladder kernel) instead of the masked tiles
+use_ladder_maps = True
+PREFILL_MAP_DIMS = (64, 128)
+
+
+def seq_extension():
+    """The sequence-state extension (its build of the paged attention
+    kernels serves the layer-list models)."""
+    return _native_seq()
 
 
 SCAN_CHUNK = 64  # rows per chunk of the chunk-parallel recurrent prefill

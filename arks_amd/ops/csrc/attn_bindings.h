@@ -24,14 +24,16 @@ void arks_attn_extend_paged(void* out, const void* q, const void* k_cache,
                             const void* tile_info, int ntiles, float scale,
                             int num_q_heads, int num_kv_heads, int head_dim,
                             int max_blocks, int64_t q_stride, int kv_fp8,
-                            int window, int sink, hipStream_t stream);
+                            int window, int sink, int maps,
+                            hipStream_t stream);
 void arks_attn_extend_paged2(void* out, const void* q, const void* k_cache,
                              const void* v_cache, const void* block_tables,
                              const void* kv_lens, const void* cu_seqlens_q,
                              const void* tile_info, void* part_ws, int ntiles,
                              float scale, int num_q_heads, int num_kv_heads,
                              int head_dim, int max_blocks, int64_t q_stride,
-                             int window, int sink, hipStream_t stream);
+                             int window, int sink, int maps,
+                             hipStream_t stream);
 void arks_attn_extend2_combine(void* out, const void* part_ws,
                                const void* combine_table,
                                const void* cu_seqlens_q, int n_split,
@@ -106,7 +108,8 @@ inline void attention_extend_paged(torch::Tensor out, torch::Tensor q,
                             torch::Tensor k_cache, torch::Tensor v_cache,
                             torch::Tensor block_tables, torch::Tensor kv_lens,
                             torch::Tensor cu_seqlens_q, torch::Tensor tile_info,
-                            double scale, int64_t window, int64_t sink) {
+                            double scale, int64_t window, int64_t sink,
+                            int64_t maps) {
   check_bf16_contig(out, "out");
   check_bf16_rowstrided(q, "q");
   const bool kv_fp8 = check_kv_cache(k_cache, "k_cache");
@@ -118,7 +121,13 @@ inline void attention_extend_paged(torch::Tensor out, torch::Tensor q,
   TORCH_CHECK(tile_info.dim() == 2 && tile_info.size(1) == 2);
   const int num_q_heads = q.size(1);
   const int head_dim = q.size(2);
-  const int num_kv_heads = k_cache.size(1);
+  // key groups: every head of the cache once per key map of its rows
+  const int num_kv_heads = k_cache.size(1) * maps;
+  TORCH_CHECK(maps >= 1 && k_cache.size(3) == head_dim * maps &&
+                  v_cache.size(3) == head_dim &&
+                  v_cache.size(1) == k_cache.size(1) &&
+                  num_q_heads % num_kv_heads == 0,
+              "cache rows do not fit the heads and key maps");
   TORCH_CHECK(k_cache.size(2) == 16, "KV block size must be 16");
   TORCH_CHECK(head_dim == 32 || head_dim == 64 || head_dim == 96 ||
                   head_dim == 128 || head_dim == 256,
@@ -133,14 +142,15 @@ inline void attention_extend_paged(torch::Tensor out, torch::Tensor q,
                          tile_info.data_ptr(), ntiles, (float)scale,
                          num_q_heads, num_kv_heads, head_dim, max_blocks,
                          q.stride(0), kv_fp8 ? 1 : 0, (int)window, (int)sink,
-                         attn_current_stream());
+                         (int)maps, attn_current_stream());
 }
 inline void attention_extend_paged2(torch::Tensor out, torch::Tensor q,
                              torch::Tensor k_cache, torch::Tensor v_cache,
                              torch::Tensor block_tables, torch::Tensor kv_lens,
                              torch::Tensor cu_seqlens_q,
                              torch::Tensor tile_info, torch::Tensor part_ws,
-                             double scale, int64_t window, int64_t sink) {
+                             double scale, int64_t window, int64_t sink,
+                             int64_t maps) {
   check_bf16_contig(out, "out");
   check_bf16_rowstrided(q, "q");
   check_bf16_contig(k_cache, "k_cache");
@@ -153,7 +163,12 @@ inline void attention_extend_paged2(torch::Tensor out, torch::Tensor q,
               "tile_info rows are (seq, q0, part, nparts)");
   const int num_q_heads = q.size(1);
   const int head_dim = q.size(2);
-  const int num_kv_heads = k_cache.size(1);
+  const int num_kv_heads = k_cache.size(1) * maps;
+  TORCH_CHECK(maps >= 1 && k_cache.size(3) == head_dim * maps &&
+                  v_cache.size(3) == head_dim &&
+                  v_cache.size(1) == k_cache.size(1) &&
+                  num_q_heads % num_kv_heads == 0,
+              "cache rows do not fit the heads and key maps");
   TORCH_CHECK(k_cache.size(2) == 16, "KV block size must be 16");
   TORCH_CHECK(head_dim == 64 || head_dim == 128, "head_dim must be 64 or 128");
   const int ntiles = tile_info.size(0);
@@ -169,7 +184,8 @@ inline void attention_extend_paged2(torch::Tensor out, torch::Tensor q,
                           kv_lens.data_ptr(), cu_seqlens_q.data_ptr(),
                           tile_info.data_ptr(), ws, ntiles, (float)scale,
                           num_q_heads, num_kv_heads, head_dim, max_blocks,
-                          q.stride(0), (int)window, (int)sink, attn_current_stream());
+                          q.stride(0), (int)window, (int)sink, (int)maps,
+                          attn_current_stream());
 }
 inline void attention_extend2_combine(torch::Tensor out, torch::Tensor part_ws,
                                torch::Tensor combine_table,

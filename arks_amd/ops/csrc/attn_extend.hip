@@ -58,7 +58,10 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
     const int* __restrict__ tile_info,     // [ntiles, 2] = (seq_idx, q0)
     const float scale, const int num_q_heads, const int num_kv_heads,
     const int max_blocks, const int64_t q_stride, const int window,
-    const int sink) {
+    const int sink,
+    // keys per cache row (see attn_extend2.hip): key group g reads key
+    // g % maps of the rows of head g / maps, whose value all maps share
+    const int maps) {
   constexpr int CHUNKS = HEAD_DIM / 16;
   constexpr int STEPS = HEAD_DIM / 32;
   // The XOR swizzle of K rows flips byte bits 4..6: it stays inside a row
@@ -124,16 +127,16 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
   for (int j = j0; j < ntiles; ++j) {
     const int key_base = j * EXT_KTILE;
     // Page base offsets for this tile's two 16-key pages.
-    const int64_t page_elems = (int64_t)num_kv_heads * PAGE * HEAD_DIM;
+    const int64_t page_rows = (int64_t)(num_kv_heads / maps) * PAGE;
+    const int64_t kstride = (int64_t)maps * HEAD_DIM;
+    const int kcol = (kvh % maps) * HEAD_DIM;
     // window-dropped pages carry block-table entry -1; their tokens are
     // masked, so the page id is sanitized to 0
     const int pg0 = max(0, bt[key_base / PAGE]);
     const int pg1 =
         (key_base + PAGE < kmax) ? max(0, bt[key_base / PAGE + 1]) : pg0;
-    const int64_t pbase0 =
-        (int64_t)pg0 * page_elems + (int64_t)kvh * PAGE * HEAD_DIM;
-    const int64_t pbase1 =
-        (int64_t)pg1 * page_elems + (int64_t)kvh * PAGE * HEAD_DIM;
+    const int64_t prow0 = (int64_t)pg0 * page_rows + (int64_t)(kvh / maps) * PAGE;
+    const int64_t prow1 = (int64_t)pg1 * page_rows + (int64_t)(kvh / maps) * PAGE;
     {
       const int nvec = EXT_KTILE * HEAD_DIM / 8;
       for (int i = tid; i < nvec; i += 256) {
@@ -142,11 +145,12 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
         const int kg = key_base + key;
         ushort8 kv{}, vv{};
         if (kg < kmax) {
-          const int64_t src = (key < PAGE ? pbase0 : pbase1) +
-                              (int64_t)(kg % PAGE) * HEAD_DIM + col8;
+          const int64_t row = (key < PAGE ? prow0 : prow1) + (kg % PAGE);
+          const int64_t ksrc = row * kstride + kcol + col8;
+          const int64_t src = row * HEAD_DIM + col8;
           if constexpr (KV_FP8) {
             uchar8 k8 = *reinterpret_cast<const uchar8*>(
-                reinterpret_cast<const uint8_t*>(k_cache) + src);
+                reinterpret_cast<const uint8_t*>(k_cache) + ksrc);
             uchar8 v8 = *reinterpret_cast<const uchar8*>(
                 reinterpret_cast<const uint8_t*>(v_cache) + src);
 #pragma unroll
@@ -155,7 +159,7 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
               vv[e] = ext_fp8_to_bf16(v8[e]);
             }
           } else {
-            kv = *reinterpret_cast<const ushort8*>(k_cache + src);
+            kv = *reinterpret_cast<const ushort8*>(k_cache + ksrc);
             vv = *reinterpret_cast<const ushort8*>(v_cache + src);
           }
         }
@@ -292,7 +296,7 @@ extern "C" void arks_attn_extend_paged(
     const void* block_tables, const void* kv_lens, const void* cu_seqlens_q,
     const void* tile_info, int ntiles, float scale, int num_q_heads,
     int num_kv_heads, int head_dim, int max_blocks, int64_t q_stride,
-    int kv_fp8, int window, int sink, hipStream_t stream) {
+    int kv_fp8, int window, int sink, int maps, hipStream_t stream) {
   dim3 grid(num_q_heads, ntiles), block(256);
 #define ARKS_EXT(D, F8)                                                       \
   hipLaunchKernelGGL((attn_extend_kernel<D, F8>), grid, block, 0, stream,     \
@@ -300,7 +304,7 @@ extern "C" void arks_attn_extend_paged(
                      (const bf16*)v_cache, (const int*)block_tables,          \
                      (const int*)kv_lens, (const int*)cu_seqlens_q,           \
                      (const int*)tile_info, scale, num_q_heads, num_kv_heads, \
-                     max_blocks, q_stride, window, sink)
+                     max_blocks, q_stride, window, sink, maps)
   if (head_dim == 128 && kv_fp8) ARKS_EXT(128, true);
   else if (head_dim == 64 && kv_fp8) ARKS_EXT(64, true);
   else if (head_dim == 128) ARKS_EXT(128, false);

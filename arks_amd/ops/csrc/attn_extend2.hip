@@ -75,7 +75,12 @@ __global__ __launch_bounds__(512) void attn_extend2_kernel(
     float* __restrict__ part_ws,  // [ntiles, Hq, QTILE, D+2] f32 slabs
     const float scale, const int num_q_heads, const int num_kv_heads,
     const int max_blocks, const int64_t q_stride, const int window,
-    const int sink) {
+    const int sink,
+    // keys per cache row: a key row holds `maps` keys of D dims side by
+    // side that share the row's value (k_cache [nblocks, Hkv / maps, 16,
+    // maps * D], v_cache [nblocks, Hkv / maps, 16, D]); key group g reads
+    // key g % maps of the rows of head g / maps
+    const int maps) {
   constexpr int STEPS = HEAD_DIM / 16;   // QK^T K-contraction steps
   constexpr int DTILES = HEAD_DIM / 32;  // 32-dim output tiles
   constexpr int CB = HEAD_DIM / 16;      // 16-col blocks per key row
@@ -155,8 +160,10 @@ __global__ __launch_bounds__(512) void attn_extend2_kernel(
   // vec8 per thread at D=64).
   constexpr int NVEC = E2_KVBLK * HEAD_DIM / 8;
   constexpr int VPT = NVEC / 512;
-  const int64_t page_elems = (int64_t)num_kv_heads * E2_PAGE * HEAD_DIM;
-  const int64_t head_off = (int64_t)kvh * E2_PAGE * HEAD_DIM;
+  const int64_t page_rows = (int64_t)(num_kv_heads / maps) * E2_PAGE;
+  const int64_t head_row = (int64_t)(kvh / maps) * E2_PAGE;
+  const int64_t kstride = (int64_t)maps * HEAD_DIM;
+  const int kcol = (kvh % maps) * HEAD_DIM;
 
   // Branchy per-element guards de-pipeline global loads (guide §5 trap (c)),
   // so full in-range tiles take an unguarded path; only the final (ragged)
@@ -171,10 +178,11 @@ __global__ __launch_bounds__(512) void attn_extend2_kernel(
         const int col8 = (e % (HEAD_DIM / 8)) * 8;
         const int kg = key_base + key;
         const int64_t pg = max(0, bt[kg / E2_PAGE]);
-        const int64_t src = pg * page_elems + head_off +
-                            (int64_t)(kg % E2_PAGE) * HEAD_DIM + col8;
-        kr[vv] = *reinterpret_cast<const ushort8*>(k_cache + src);
-        vr[vv] = *reinterpret_cast<const ushort8*>(v_cache + src);
+        const int64_t row = pg * page_rows + head_row + (kg % E2_PAGE);
+        kr[vv] = *reinterpret_cast<const ushort8*>(k_cache + row * kstride +
+                                                   kcol + col8);
+        vr[vv] = *reinterpret_cast<const ushort8*>(v_cache + row * HEAD_DIM +
+                                                   col8);
       }
       return;
     }
@@ -189,10 +197,11 @@ __global__ __launch_bounds__(512) void attn_extend2_kernel(
         // window-dropped pages are -1 in the block table; sanitized to 0
         // (their tokens are masked out)
         const int64_t pg = max(0, bt[kg / E2_PAGE]);
-        const int64_t src = pg * page_elems + head_off +
-                            (int64_t)(kg % E2_PAGE) * HEAD_DIM + col8;
-        kv = *reinterpret_cast<const ushort8*>(k_cache + src);
-        vv8 = *reinterpret_cast<const ushort8*>(v_cache + src);
+        const int64_t row = pg * page_rows + head_row + (kg % E2_PAGE);
+        kv = *reinterpret_cast<const ushort8*>(k_cache + row * kstride +
+                                               kcol + col8);
+        vv8 = *reinterpret_cast<const ushort8*>(v_cache + row * HEAD_DIM +
+                                                col8);
       }
       kr[vv] = kv;
       vr[vv] = vv8;
@@ -486,7 +495,7 @@ extern "C" void arks_attn_extend_paged2(
     const void* block_tables, const void* kv_lens, const void* cu_seqlens_q,
     const void* tile_info, void* part_ws, int ntiles, float scale,
     int num_q_heads, int num_kv_heads, int head_dim, int max_blocks,
-    int64_t q_stride, int window, int sink, hipStream_t stream) {
+    int64_t q_stride, int window, int sink, int maps, hipStream_t stream) {
   dim3 grid(num_q_heads, ntiles), block(512);
   static bool attr_set[2] = {false, false};
   auto launch = [&](auto kern, int lds_bytes, int idx) {
@@ -502,7 +511,7 @@ extern "C" void arks_attn_extend_paged2(
                        (const int*)kv_lens, (const int*)cu_seqlens_q,
                        (const int*)tile_info, (float*)part_ws, scale,
                        num_q_heads, num_kv_heads, max_blocks, q_stride,
-                       window, sink);
+                       window, sink, maps);
   };
   if (head_dim == 128) {
     constexpr int LDS = (2 * 64 * 128 + 2 * 16 * 8 * VBLK_ELEMS) * 2;

@@ -334,6 +334,30 @@ def test_fast_path_sizes(tmp_path, device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", GPU_CASES)
+def test_long_portions_beside_single_rows(tmp_path, device, dtype):
+    """Steps whose longest portion fills a 256-row tile take the work-sorted
+    prefill kernels for the two-map layers too: a first portion, a portion
+    over a cached prefix, and single rows of another request in the same
+    steps."""
+    cfg = O.make_config(
+        [D(heads=4, kv_heads=2, dim=64, vdim=64, conv=4, every=50, mlp=None),
+         D(heads=4, kv_heads=2, dim=64, vdim=64, conv=4, every=50, kv_from=0,
+           mlp=None),
+         D(heads=2, kv_heads=1, dim=128, vdim=128, conv=3, mlp=MOE(top=6))],
+        width=64)
+    w = write_checkpoint(tmp_path / "m", cfg)
+    ta, tb = toks(600, seed=13), toks(280, seed=14)
+    eng = make_engine(tmp_path / "m", device, dtype, max_tokens=1024)
+    steps = [[("a", ta[:300], False)],
+             [("a", ta[300:301], False), ("b", tb[:270], False)],
+             [("a", ta[301:561], False), ("b", tb[270:271], False)],
+             [("a", ta[561:], True), ("b", tb[271:], True)]]
+    got = replay(eng, tmp_path, steps)
+    assert_logits(got["a"], cfg, w, ta, dtype)
+    assert_logits(got["b"], cfg, w, tb, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", GPU_CASES)
 def test_key_valued_head_sizes(tmp_path, device, dtype):
     """Every head size the matrix-core kernels of plain causal attention are
     built for, with the vectorised turn-and-norm kernel where the size
@@ -466,8 +490,8 @@ class MapPages:
     scrambled order, and steps of rows over them through
     ops.attention_sink_paged(maps=2)."""
 
-    def __init__(self, dev, dtype, G, Dk, V, n):
-        self.dev, self.dt = dev, TDT[dtype]
+    def __init__(self, dev, dtype, G, Dk, V, n, ladder=False):
+        self.dev, self.dt, self.ladder = dev, TDT[dtype], ladder
         nblk = -(-n // 16)
         g = torch.Generator().manual_seed(7)
         self.table = torch.randperm(nblk + 3, generator=g)[:nblk].to(torch.int32)
@@ -486,12 +510,22 @@ class MapPages:
         self.k[blk, :, off] = k.reshape(n, G, 2 * Dk).to(self.dt).to(self.dev)
         self.v[blk, :, off] = v.to(self.dt).to(self.dev)
         self.len += n
-        out = ops.attention_sink_paged(
-            q.reshape(n, G * 2 * R, Dk).to(self.dt).to(self.dev).contiguous(),
-            self.k, self.v, self.table[None].to(self.dev),
-            _i32([self.len], self.dev), _i32([0, n], self.dev),
-            _i32([0] * n, self.dev), scale, False, None, False, n,
-            pos.to(self.dev), maps=2)
+        qd = q.reshape(n, G * 2 * R, Dk).to(self.dt).to(self.dev).contiguous()
+        if self.ladder and n > 1:
+            # the work-sorted prefill kernels (bf16, 64 / 128 wide heads)
+            tiles = ops.build_extend_tiles([n], [self.len], False, self.dev,
+                                           num_q_heads=G * 2 * R,
+                                           flash_decode=False)
+            out = ops.attention_extend_paged(
+                qd, self.k, self.v, self.table[None].to(self.dev),
+                _i32([self.len], self.dev), _i32([0, n], self.dev), None,
+                scale, tiles=tiles, native=ops.seq_extension(), maps=2)
+        else:
+            out = ops.attention_sink_paged(
+                qd, self.k, self.v, self.table[None].to(self.dev),
+                _i32([self.len], self.dev), _i32([0, n], self.dev),
+                _i32([0] * n, self.dev), scale, False, None, False, n,
+                pos.to(self.dev), maps=2)
         return out.double().cpu().view(n, G, 2, R, -1)
 
 
@@ -533,6 +567,38 @@ def test_one_key_wins_in_one_map_only(device, dtype, decode, Dk, V):
         got = pg.step(q[cut:], k[cut:], v[cut:], 0.5)[-1]
         tol = 1e-4 if dtype == "float32" else 2e-2
         assert torch.allclose(got, want, atol=tol, rtol=tol), (hot, hot_map)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("Dk", [64, 128])
+def test_two_map_prompts_on_the_prefill_kernels(Dk):
+    """Prompt portions over two-map rows through the 256-row ladder and the
+    64-row kernels: a first portion of 300 rows, a second of 130 over it, a
+    third of 40; against the oracle and against the masked tile kernel. One
+    key per map carries a huge score for the last row."""
+    dev = torch.device("cuda")
+    G, R, V, n = 2, 2, Dk, 470
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn(n, G, 2, R, Dk, generator=g, dtype=F64)
+    k = torch.randn(n, G, 2, Dk, generator=g, dtype=F64)
+    v = _rounded(torch.randn(n, G, V, generator=g, dtype=F64), "bfloat16")
+    q[n - 1] *= 0.0
+    q[n - 1, ..., 5] = 9.0
+    k[7, :, 0, 5], k[301, :, 1, 5] = 30.0, 30.0
+    q, k = _rounded(q, "bfloat16"), _rounded(k, "bfloat16")
+    scale = Dk ** -0.5
+    want = torch.stack([
+        O.softmax_attend(q[:, :, m].reshape(n, G * R, Dk), k[:, :, m], v, scale)
+        for m in (0, 1)], 0).view(2, n, G, R, V).permute(1, 2, 0, 3, 4)
+    assert torch.allclose(want[n - 1, 0, 0, 0], v[7, 0], atol=1e-6)
+    assert torch.allclose(want[n - 1, 1, 1, 1], v[301, 1], atol=1e-6)
+    got = {}
+    for ladder in (True, False):
+        pg = MapPages(dev, "bfloat16", G, Dk, V, n, ladder=ladder)
+        got[ladder] = torch.cat([pg.step(q[a:b], k[a:b], v[a:b], scale)
+                                 for a, b in [(0, 300), (300, 430), (430, 470)]])
+        assert torch.allclose(got[ladder], want, atol=2e-2, rtol=2e-2), ladder
+    assert torch.allclose(got[True], got[False], atol=2e-2, rtol=2e-2)
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
