@@ -152,8 +152,9 @@ class ModelConfig:
 class HybridModelConfig:
     """Layer-list decoders: config.json names one architecture and lists the
     layers, each with its mixer type ("attention", "lightning", "mamba1",
-    "parallel"), the mixer's sizes and an optional feed-forward (dense, or
-    "moe" where the architecture has one). Every size and every
+    "parallel", "latent_attention", "mamba2", "attention_2": what a type
+    means is the architecture's), the mixer's sizes and an optional
+    feed-forward (dense, or "moe" where the architecture has one). Every size and every
     per-model constant comes from that file; what the architecture itself
     fixes (block arrangement, activation, rotary pairing) lives with the
     model code (arks_amd/models/hybrid.py)."""

@@ -68,10 +68,10 @@ def main():
         t256 = tiles256([qlen] * S, [kvlen] * S, "cuda")
         nat = ops._native()
         t_old = bench(lambda: nat.attention_extend_paged(
-            out, q, kc, vc, bt, kvl, cu, t64i, scale, 0))
+            out, q, kc, vc, bt, kvl, cu, t64i, scale, 0, 0, 1))
         ws0 = torch.empty(0, dtype=torch.float32, device="cuda")
         t_new = bench(lambda: nat.attention_extend_paged2(
-            out, q, kc, vc, bt, kvl, cu, t256, ws0, scale, 0))
+            out, q, kc, vc, bt, kvl, cu, t256, ws0, scale, 0, 0, 1))
         # split path: prebuilt tiles (as the engine does once per batch)
         tiles = ops.build_extend_tiles([qlen] * S, [kvlen] * S, False,
                                        "cuda", num_q_heads=hq)

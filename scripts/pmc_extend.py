@@ -35,7 +35,7 @@ def main():
     nat = ops._native()
     for _ in range(20):
         nat.attention_extend_paged2(out, q, kc, vc, bt, kvl, cu, t256, ws0,
-                                    1.0 / math.sqrt(hd), 0)
+                                    1.0 / math.sqrt(hd), 0, 0, 1)
     torch.cuda.synchronize()
 
 
